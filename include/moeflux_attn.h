@@ -1,0 +1,261 @@
+/*
+ * moeflux_attn.h — C ABI of the MI355X (gfx950) attention path for moeflux.
+ *
+ * The library replaces, for the attention core of each layer, what the Rust
+ * host of mdegans/moeflux hands to metal-rs: the four full-attention kernels
+ * and the five Gated-DeltaNet kernels, together with the per-layer state they
+ * read and write (KV cache, conv state, recurrent state).  Each declaration
+ * cites the reference interface it stands in for.  Conventions are those of
+ * the reference's own C API (crates/moeflux-sys/metal_infer/moeflux.h:9-11,
+ * 38, 52-64, 177-182): an opaque context first, int32_t shapes, caller-owned
+ * buffers, 0 on success and a negative code on error, NULL from create on
+ * failure, destroy(NULL) is a no-op.  A context is single-threaded
+ * (crates/moeflux/src/lib.rs:22-27); two contexts may be used concurrently.
+ *
+ * Host-pointer entry points are synchronous at return.  `_dev` entry points
+ * take device pointers, enqueue on the context's HIP stream and return; pair
+ * them with mfa_sync().
+ */
+#ifndef MOEFLUX_ATTN_H
+#define MOEFLUX_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Every declaration below is an exported symbol of libmoeflux_attn_hip.so. */
+#pragma GCC visibility push(default)
+
+typedef struct mfa_ctx mfa_ctx;
+
+/* Error codes.  The reference collapses every failure to -1
+ * (moeflux.h:177-178, 473-474); this library keeps "negative means failure"
+ * and distinguishes the classes the Rust side maps to typed errors
+ * (SdpaError sdpa.rs:41-55, LinearAttnError linear_attn.rs:29-54,
+ * GpuAttnError gpu_attn.rs:46-63). */
+#define MFA_OK 0
+#define MFA_ERR_INVALID (-1)  /* NULL pointer, non-positive shape, kv_len <= 0, divisibility */
+#define MFA_ERR_SHAPE (-2)    /* valid but unsupported by the kernels (head_dim, key_dim ...) */
+#define MFA_ERR_OVERFLOW (-3) /* KV append past capacity (full_attn_forward.rs:283-288) */
+#define MFA_ERR_LAYER (-4)    /* layer index out of range or of the other kind */
+#define MFA_ERR_HIP (-5)      /* a HIP runtime call failed; see mfa_last_error_string() */
+#define MFA_ERR_STATE (-6)    /* snapshot does not match this context (state_snapshot.rs preflight) */
+
+#define MFA_KV_F32 0
+#define MFA_KV_BF16 1
+
+/* Shapes are run-time values, as the reference's kernel arguments are
+ * (NOTES.md:92-103); they mirror the fields of `Variant`
+ * (crates/moeflux/src/riir/variants.rs:383-465). */
+typedef struct mfa_config {
+    int32_t num_layers;
+    int32_t full_attn_interval;  /* layer i is full attention iff (i+1) % interval == 0 (variants.rs:258-264) */
+    int32_t num_attn_heads;
+    int32_t num_kv_heads;
+    int32_t head_dim;            /* 64, 128 or 256 */
+    int32_t kv_capacity;         /* positions per full-attention layer (reference: GPU_KV_SEQ / MAX_SEQ_LEN, variants.rs:377-379) */
+    int32_t kv_dtype;            /* MFA_KV_F32 or MFA_KV_BF16 */
+    int32_t linear_num_k_heads;
+    int32_t linear_num_v_heads;
+    int32_t linear_key_dim;      /* 128 (variants.rs:219-223) */
+    int32_t linear_value_dim;    /* 128 */
+    int32_t conv_kernel_size;    /* 4 */
+    float rms_norm_eps;          /* 1e-6 (variants.rs:358) */
+} mfa_config;
+
+/* ---- lifecycle ----------------------------------------------------------- */
+
+/* Replaces RsCtx::open's state allocation (riir/mod.rs:270-318,
+ * state.rs:400-413) and LayerForwardBuffers::new (linear_attn_forward.rs:
+ * 180-244) for the attention state: allocates, zero-filled, one KV cache per
+ * full-attention layer and one conv + recurrent state per linear layer, plus
+ * the split-K workspace and one HIP stream.  NULL on failure. */
+mfa_ctx *mfa_ctx_create(const mfa_config *cfg);
+/* moeflux.h:62-64 (mf_free_model).  No-op on NULL. */
+void mfa_ctx_destroy(mfa_ctx *ctx);
+/* Text of the last error on the calling thread ("" if none). */
+const char *mfa_last_error_string(void);
+/* Block until everything enqueued on the context's stream has finished. */
+int mfa_sync(mfa_ctx *ctx);
+/* The context's hipStream_t, for callers that enqueue their own work around
+ * the `_dev` calls. */
+void *mfa_stream(mfa_ctx *ctx);
+
+/* Per-layer constants of a linear-attention layer, read by the reference from
+ * the weight file inside each call (linear_attn_forward.rs:607-664 passes
+ * conv1d.weight, A_log, dt_bias, norm.weight offsets).  Host pointers, copied.
+ *   conv_w_bf16 [C*K] channel-major, a_log f32 [Hv], dt_bias_bf16 [Hv],
+ *   norm_w_bf16 [dv]. */
+int mfa_set_linear_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *conv_w_bf16,
+                           const float *a_log, const uint16_t *dt_bias_bf16,
+                           const uint16_t *norm_w_bf16);
+
+/* Override the split-K partition count of the decode kernel (0 = automatic).
+ * The result must not depend on it; tests use it to check exactly that, as
+ * the reference checks tiled against single-shot MLA (tests/mla_sdpa_tiled.rs:
+ * 176-216). */
+int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits);
+
+/* ---- full attention: production path -------------------------------------- */
+
+/* Replaces the KV append of full_attn_forward.rs:282-323 (host cache row +
+ * GPU mirror row).  k, v: [num_kv_heads*head_dim] f32 host rows (K post-norm
+ * post-RoPE, V raw).  MFA_ERR_OVERFLOW when the layer is full. */
+int mfa_kv_append(mfa_ctx *ctx, int32_t layer, const float *k, const float *v);
+int mfa_kv_append_dev(mfa_ctx *ctx, int32_t layer, const float *k_dev, const float *v_dev);
+/* KvCache::len (state.rs:37-41). */
+int32_t mfa_kv_len(mfa_ctx *ctx, int32_t layer);
+
+/* Replaces both branches of full_attn_forward.rs:331-389: the four-kernel GPU
+ * chain attn_scores_batched / attn_softmax_batched / attn_values_batched /
+ * sigmoid_gate (linear_attn_forward.rs:850-902) and the sdpa_cpu fallback
+ * (sdpa.rs:63-172), at every kv_len >= 1.  q, q_gate, out: [Hq*head_dim] f32. */
+int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_gate,
+                    float *out);
+int mfa_sdpa_decode_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev,
+                        const float *q_gate_dev, float *out_dev);
+
+/* A chunk of T prompt tokens on one full-attention layer.  The reference has
+ * no batched prefill: eval_prompt is a token loop (riir/mod.rs:1196-1214); the
+ * result equals T successive mfa_kv_append + mfa_sdpa_decode calls.
+ *   q, q_gate, out: [T, Hq*head_dim]; k, v: [T, num_kv_heads*head_dim]. */
+int mfa_prefill_attn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q,
+                     const float *q_gate, const float *k, const float *v, float *out);
+int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_dev,
+                         const float *q_gate_dev, const float *k_dev, const float *v_dev,
+                         float *out_dev);
+
+/* ---- Gated DeltaNet: production path -------------------------------------- */
+
+/* Replaces the five-kernel chain conv1d_step, rms_norm_qk, compute_decay_beta,
+ * gated_delta_net_step, gated_rms_norm encoded at linear_attn_forward.rs:
+ * 607-664 (encoders gpu_linear_attn.rs:54-202).  qkv_in [C] = [q|k|v] f32 with
+ * C = 2*Hk*dk + Hv*dv; z, out [Hv*dv]; alpha, beta [Hv].  Advances the
+ * layer's conv state and recurrent state. */
+int mfa_gdn_step(mfa_ctx *ctx, int32_t layer, const float *qkv_in, const float *z,
+                 const float *alpha, const float *beta, float *out);
+int mfa_gdn_step_dev(mfa_ctx *ctx, int32_t layer, const float *qkv_in_dev,
+                     const float *z_dev, const float *alpha_dev, const float *beta_dev,
+                     float *out_dev);
+
+/* T prompt tokens on one linear layer; equals T successive mfa_gdn_step calls
+ * (riir/mod.rs:1196-1214).  Inputs are [T, ...] row-major. */
+int mfa_prefill_gdn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv_in,
+                    const float *z, const float *alpha, const float *beta, float *out);
+int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv_in_dev,
+                        const float *z_dev, const float *alpha_dev, const float *beta_dev,
+                        float *out_dev);
+
+/* ---- one token's attention launches over the whole stack ------------------ */
+
+/* The attention work of one step_internal layer loop (riir/mod.rs:1769-1888):
+ * for each layer in order, mfa_sdpa_decode_dev or mfa_gdn_step_dev on that
+ * layer's slice of the inputs.  Inputs are packed per kind, in layer order:
+ *   full_q, full_gate, full_out: [n_full, Hq*head_dim];
+ *   lin_qkv [n_lin, C]; lin_z, lin_out [n_lin, Hv*dv]; lin_alpha, lin_beta [n_lin, Hv].
+ * The KV caches are used as they stand (append first). */
+int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gate,
+                        float *full_out, const float *lin_qkv, const float *lin_z,
+                        const float *lin_alpha, const float *lin_beta, float *lin_out);
+
+/* ---- state operations ------------------------------------------------------ */
+
+/* memory_clear (riir/mod.rs:1950-1969; state.rs clear_all): KV lengths to 0,
+ * caches zeroed, conv and recurrent state zeroed. */
+int mfa_reset(mfa_ctx *ctx);
+/* memory_seq_rm (state.rs:431-455): every KV cache keeps positions
+ * [0, min(max(p0,0), p1<0 ? len : min(p1,len))) and the dropped rows are
+ * zero-filled; every linear layer is reset (lossy, as in the reference). */
+int mfa_truncate(mfa_ctx *ctx, int32_t p0, int32_t p1);
+/* memory_seq_pos_max (state.rs:457-473): largest KV length, -1 if the stack
+ * has no full-attention layer. */
+int32_t mfa_pos_max(mfa_ctx *ctx);
+
+/* Per-layer state in the reference's host layouts (the buffers
+ * state_snapshot.rs:16-27 serialises).  KV rows are [len, num_kv_heads*head_dim]
+ * f32 (a bf16 cache widens exactly on export and rounds to nearest-even on
+ * import); conv state is [K-1, C] time-major with the newest input last;
+ * recurrent state is [Hv, dv, dk]. */
+int mfa_kv_export(mfa_ctx *ctx, int32_t layer, int32_t max_rows, float *k_out, float *v_out);
+int mfa_kv_import(mfa_ctx *ctx, int32_t layer, int32_t len, const float *k, const float *v);
+/* Same as mfa_kv_import with rows already in bf16 bits (context must be MFA_KV_BF16). */
+int mfa_kv_import_bf16(mfa_ctx *ctx, int32_t layer, int32_t len, const uint16_t *k,
+                       const uint16_t *v);
+int mfa_linear_state_export(mfa_ctx *ctx, int32_t layer, float *conv_state_out,
+                            float *ssm_state_out);
+int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state,
+                            const float *ssm_state);
+
+/* ---- timing ---------------------------------------------------------------- */
+
+/* hipEvent pair on the context's stream (the reference's counterpart is the
+ * wall-clock LayerTimingAccum, infer.m:96-114). */
+int mfa_timer_start(mfa_ctx *ctx);
+int mfa_timer_stop(mfa_ctx *ctx, float *elapsed_ms);
+
+/* ---- stateless per-kernel hooks (host pointers, synchronous) --------------- */
+/* Twins of the reference's per-kernel test hooks: each uploads its operands,
+ * runs ONE kernel, waits and copies back (gpu_attn.rs:247-416). */
+
+/* mf_sdpa_cpu (moeflux.h:179-182; RsCtx::sdpa_cpu riir/mod.rs:444) with the
+ * shape passed explicitly. */
+int mfa_sdpa(int32_t kv_len, int32_t num_attn_heads, int32_t num_kv_heads, int32_t head_dim,
+             const float *q, const float *q_gate, const float *k_cache, const float *v_cache,
+             float *out);
+/* The same over a bf16 K/V cache (rows of uint16 bf16 bits). */
+int mfa_sdpa_bf16kv(int32_t kv_len, int32_t num_attn_heads, int32_t num_kv_heads,
+                    int32_t head_dim, const float *q, const float *q_gate,
+                    const uint16_t *k_cache, const uint16_t *v_cache, float *out);
+/* mf_attn_scores_batched (moeflux.h:475-483; shaders.metal:976-1019). */
+int mfa_attn_scores_batched(int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t seq_len, const float *q, const float *k_cache, float scale,
+                            float *scores_out);
+/* mf_attn_softmax_batched (moeflux.h:494-497; shaders.metal:1026-1084). */
+int mfa_attn_softmax_batched(int32_t num_heads, int32_t seq_len, float *scores_inout);
+/* mf_attn_values_batched (moeflux.h:508-515; shaders.metal:1095-1117). */
+int mfa_attn_values_batched(int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t seq_len, const float *scores, const float *v_cache,
+                            float *out);
+/* mf_sigmoid_gate (moeflux.h:524-527; shaders.metal:1125-1134). */
+int mfa_sigmoid_gate(int32_t dim, const float *gate, float *x_inout);
+
+/* conv1d_step kernel (shaders.metal:1213-1244; encoder gpu_linear_attn.rs:54-77):
+ * out = silu(conv) AND the state is rolled in place, as the GPU kernel does.
+ * (mf_conv1d_step_cpu, moeflux.h:224-228, leaves the roll to its caller.) */
+int mfa_conv1d_step(int32_t channels, int32_t kernel_size, float *conv_state_inout,
+                    const float *new_input, const uint16_t *weight_bf16, float *out);
+/* rms_norm_qk kernel (shaders.metal:1254-1303; gpu_linear_attn.rs:82-103). In place. */
+int mfa_rms_norm_qk(int32_t num_k_heads, int32_t key_dim, float *q_inout, float *k_inout);
+/* mf_rms_norm_bare_cpu (moeflux.h:234-235; linear_attn.rs:160-184). */
+int mfa_rms_norm_bare(int32_t dim, float eps, const float *x, float *out);
+/* compute_decay_beta kernel (shaders.metal:1312-1327; gpu_linear_attn.rs:108-133). */
+int mfa_compute_decay_beta(int32_t num_v_heads, const float *alpha, const float *beta,
+                           const float *a_log, const uint16_t *dt_bias_bf16, float *g_decay_out,
+                           float *beta_gate_out);
+/* gated_delta_net_step kernel (shaders.metal:1154-1194; gpu_linear_attn.rs:140-172). */
+int mfa_gated_delta_net_step(int32_t v_heads, int32_t k_heads, int32_t key_dim,
+                             int32_t value_dim, const float *g_decay, const float *beta_gate,
+                             const float *q, const float *k, const float *v,
+                             float *ssm_state_inout, float *out_values);
+/* mf_gated_delta_recurrence_cpu (moeflux.h:266-272; linear_attn.rs:288-414) with
+ * A_log / dt_bias passed instead of looked up by layer. */
+int mfa_gated_delta_recurrence(const float *a_log, const uint16_t *dt_bias_bf16,
+                               const float *alpha, const float *beta, const float *q,
+                               const float *k, const float *v, int32_t v_heads, int32_t k_heads,
+                               int32_t key_dim, int32_t value_dim, float *ssm_state_inout,
+                               float *out_values);
+/* gated_rms_norm kernel (shaders.metal:1337-1370; gpu_linear_attn.rs:177-202;
+ * mf_rms_norm_gated_cpu moeflux.h:245-249 is the one-head case num_heads = 1).
+ * x, z, out: [num_heads*dim]; weight_bf16 [dim] shared by all heads. */
+int mfa_gated_rms_norm(int32_t num_heads, int32_t dim, float eps, const float *x,
+                       const float *z, const uint16_t *weight_bf16, float *out);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOEFLUX_ATTN_H */

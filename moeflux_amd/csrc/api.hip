@@ -1,0 +1,862 @@
+// Host side of libmoeflux_attn_hip: context, state operations and the extern "C"
+// entry points declared in include/moeflux_attn.h.
+#include <cstdarg>
+#include <cstring>
+#include <new>
+
+#include "mfa_internal.h"
+
+namespace mfa {
+
+static thread_local std::string g_last_error;
+
+void set_error(const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int full_layer(Ctx *c, int32_t layer, FullLayer **out) {
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (layer < 0 || layer >= c->cfg.num_layers)
+        return fail(MFA_ERR_LAYER, "layer %d out of range [0, %d)", layer, c->cfg.num_layers);
+    if (c->kind[layer] != 1)
+        return fail(MFA_ERR_LAYER, "layer %d is a linear-attention layer", layer);
+    *out = &c->full[c->slot[layer]];
+    return MFA_OK;
+}
+
+int linear_layer(Ctx *c, int32_t layer, LinearLayer **out) {
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (layer < 0 || layer >= c->cfg.num_layers)
+        return fail(MFA_ERR_LAYER, "layer %d out of range [0, %d)", layer, c->cfg.num_layers);
+    if (c->kind[layer] != 0)
+        return fail(MFA_ERR_LAYER, "layer %d is a full-attention layer", layer);
+    *out = &c->lin[c->slot[layer]];
+    return MFA_OK;
+}
+
+int ensure_stage(Ctx *c, size_t elems) {
+    if (elems <= c->stage_elems) return MFA_OK;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    if (c->stage) MFA_HIP(hipFree(c->stage));
+    c->stage = nullptr;
+    c->stage_elems = 0;
+    MFA_HIP(hipMalloc((void **)&c->stage, elems * sizeof(float)));
+    c->stage_elems = elems;
+    return MFA_OK;
+}
+
+static SdpaWorkspace workspace(Ctx *c) {
+    return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems};
+}
+
+static int h2d(Ctx *c, void *dst, const void *src, size_t bytes) {
+    MFA_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, c->stream));
+    return MFA_OK;
+}
+static int d2h_sync(Ctx *c, void *dst, const void *src, size_t bytes) {
+    MFA_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c->stream));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+static void destroy(Ctx *c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    for (auto &f : c->full) {
+        if (f.k) (void)hipFree(f.k);
+        if (f.v) (void)hipFree(f.v);
+    }
+    for (auto &l : c->lin) {
+        if (l.conv_ring) (void)hipFree(l.conv_ring);
+        if (l.ssm) (void)hipFree(l.ssm);
+        if (l.w.conv_w) (void)hipFree(l.w.conv_w);
+        if (l.w.a_log) (void)hipFree(l.w.a_log);
+        if (l.w.dt_bias) (void)hipFree(l.w.dt_bias);
+        if (l.w.norm_w) (void)hipFree(l.w.norm_w);
+    }
+    if (c->part_o) (void)hipFree(c->part_o);
+    if (c->part_ml) (void)hipFree(c->part_ml);
+    if (c->stage) (void)hipFree(c->stage);
+    if (c->ev0) (void)hipEventDestroy(c->ev0);
+    if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+static int validate(const mfa_config *cfg, bool *has_full, bool *has_lin) {
+    if (!cfg) return fail(MFA_ERR_INVALID, "NULL config");
+    if (cfg->num_layers <= 0 || cfg->full_attn_interval <= 0)
+        return fail(MFA_ERR_INVALID, "num_layers and full_attn_interval must be positive");
+    *has_full = false;
+    *has_lin = false;
+    for (int i = 0; i < cfg->num_layers; i++) {
+        if ((i + 1) % cfg->full_attn_interval == 0) *has_full = true;
+        else *has_lin = true;
+    }
+    if (*has_full) {
+        if (cfg->num_attn_heads <= 0 || cfg->num_kv_heads <= 0 || cfg->head_dim <= 0 ||
+            cfg->kv_capacity <= 0)
+            return fail(MFA_ERR_INVALID, "non-positive full-attention shape");
+        if (cfg->num_attn_heads % cfg->num_kv_heads != 0)
+            return fail(MFA_ERR_INVALID, "num_attn_heads %d is not a multiple of num_kv_heads %d",
+                        cfg->num_attn_heads, cfg->num_kv_heads);
+        if (!sdpa_shape_supported(cfg->kv_dtype, cfg->head_dim))
+            return fail(MFA_ERR_SHAPE, "head_dim %d / kv_dtype %d not supported (64, 128, 256; f32, bf16)",
+                        cfg->head_dim, cfg->kv_dtype);
+    }
+    if (*has_lin) {
+        if (cfg->linear_num_k_heads <= 0 || cfg->linear_num_v_heads <= 0 ||
+            cfg->linear_key_dim <= 0 || cfg->linear_value_dim <= 0 || cfg->conv_kernel_size <= 0)
+            return fail(MFA_ERR_INVALID, "non-positive linear-attention shape");
+        if (cfg->linear_num_v_heads % cfg->linear_num_k_heads != 0)
+            return fail(MFA_ERR_INVALID, "linear_num_v_heads %d is not a multiple of linear_num_k_heads %d",
+                        cfg->linear_num_v_heads, cfg->linear_num_k_heads);
+        if (!gdn_shape_supported(cfg->linear_num_k_heads, cfg->linear_num_v_heads,
+                                 cfg->linear_key_dim, cfg->linear_value_dim, cfg->conv_kernel_size))
+            return fail(MFA_ERR_SHAPE, "linear-attention shape dk=%d dv=%d K=%d not supported",
+                        cfg->linear_key_dim, cfg->linear_value_dim, cfg->conv_kernel_size);
+    }
+    return MFA_OK;
+}
+
+static int create(const mfa_config *cfg, Ctx **out) {
+    bool has_full, has_lin;
+    MFA_TRY(validate(cfg, &has_full, &has_lin));
+    int ndev = 0;
+    MFA_HIP(hipGetDeviceCount(&ndev));
+    if (ndev <= 0) return fail(MFA_ERR_HIP, "no HIP device");
+    Ctx *c = new (std::nothrow) Ctx();
+    if (!c) return fail(MFA_ERR_INVALID, "out of host memory");
+    *out = c;
+    c->cfg = *cfg;
+    MFA_HIP(hipGetDevice(&c->device));
+    hipDeviceProp_t prop;
+    MFA_HIP(hipGetDeviceProperties(&prop, c->device));
+    c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    MFA_HIP(hipStreamCreate(&c->stream));
+    MFA_HIP(hipEventCreate(&c->ev0));
+    MFA_HIP(hipEventCreate(&c->ev1));
+    c->kind.resize(cfg->num_layers);
+    c->slot.resize(cfg->num_layers);
+    int nfull = 0, nlin = 0;
+    for (int i = 0; i < cfg->num_layers; i++) {
+        const bool full = (i + 1) % cfg->full_attn_interval == 0;  // variants.rs:258-264
+        c->kind[i] = full ? 1 : 0;
+        c->slot[i] = full ? nfull++ : nlin++;
+    }
+    c->full.resize(nfull);
+    c->lin.resize(nlin);
+    if (nfull) {
+        const int blk = cfg->kv_dtype == MFA_KV_BF16 ? 32 : 16;
+        c->cap_pad = ((int64_t)cfg->kv_capacity + blk - 1) / blk * blk;
+        c->plane_elems = (size_t)c->cap_pad * cfg->head_dim;
+        const size_t bytes = c->plane_elems * cfg->num_kv_heads * c->kv_elem_size();
+        for (auto &f : c->full) {
+            MFA_HIP(hipMalloc(&f.k, bytes));
+            MFA_HIP(hipMalloc(&f.v, bytes));
+            MFA_HIP(hipMemsetAsync(f.k, 0, bytes, c->stream));
+            MFA_HIP(hipMemsetAsync(f.v, 0, bytes, c->stream));
+        }
+        int splits = sdpa_pick_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
+                                      cfg->head_dim, cfg->kv_capacity, c->num_cus, 0);
+        if (splits < 128) splits = 128;
+        c->part_o_elems = sdpa_workspace_o_elems(cfg->num_attn_heads, cfg->num_kv_heads, cfg->head_dim, splits);
+        c->part_ml_elems = sdpa_workspace_ml_elems(cfg->num_attn_heads, cfg->num_kv_heads, splits);
+        MFA_HIP(hipMalloc((void **)&c->part_o, c->part_o_elems * sizeof(float)));
+        MFA_HIP(hipMalloc((void **)&c->part_ml, c->part_ml_elems * sizeof(float)));
+    }
+    if (nlin) {
+        const size_t C = (size_t)c->conv_dim(), K = (size_t)cfg->conv_kernel_size;
+        const size_t ssm = (size_t)cfg->linear_num_v_heads * cfg->linear_value_dim * cfg->linear_key_dim;
+        const int Hv = cfg->linear_num_v_heads;
+        for (auto &l : c->lin) {
+            MFA_HIP(hipMalloc((void **)&l.conv_ring, K * C * sizeof(float)));
+            MFA_HIP(hipMalloc((void **)&l.ssm, ssm * sizeof(float)));
+            MFA_HIP(hipMemsetAsync(l.conv_ring, 0, K * C * sizeof(float), c->stream));
+            MFA_HIP(hipMemsetAsync(l.ssm, 0, ssm * sizeof(float), c->stream));
+            MFA_HIP(hipMalloc((void **)&l.w.conv_w, C * K * 2));
+            MFA_HIP(hipMalloc((void **)&l.w.a_log, Hv * sizeof(float)));
+            MFA_HIP(hipMalloc((void **)&l.w.dt_bias, Hv * 2));
+            MFA_HIP(hipMalloc((void **)&l.w.norm_w, (size_t)cfg->linear_value_dim * 2));
+        }
+    }
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+static int reset_linear(Ctx *c, LinearLayer &l) {
+    const size_t C = (size_t)c->conv_dim(), K = (size_t)c->cfg.conv_kernel_size;
+    const size_t ssm = (size_t)c->cfg.linear_num_v_heads * c->cfg.linear_value_dim * c->cfg.linear_key_dim;
+    MFA_HIP(hipMemsetAsync(l.conv_ring, 0, K * C * sizeof(float), c->stream));
+    MFA_HIP(hipMemsetAsync(l.ssm, 0, ssm * sizeof(float), c->stream));
+    l.step = 0;
+    return MFA_OK;
+}
+
+// KvCache::truncate (state.rs:60-74): no-op unless 0 <= new_len <= len; zero the dropped rows.
+static int truncate_full(Ctx *c, FullLayer &f, int32_t new_len) {
+    if (new_len < 0 || new_len > f.len) return MFA_OK;
+    if (new_len < f.len)
+        MFA_TRY(launch_kv_zero(c->stream, c->cfg.kv_dtype, c->cfg.num_kv_heads, c->cfg.head_dim,
+                               c->plane_elems, new_len, f.len, f.k, f.v));
+    f.len = new_len;
+    return MFA_OK;
+}
+
+static int sdpa_decode_dev(Ctx *c, FullLayer *f, const float *q, const float *gate, float *out) {
+    if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
+    return launch_sdpa_decode(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
+                              c->cfg.head_dim, f->len, c->plane_elems, f->k, f->v, q, gate, out,
+                              workspace(c), c->num_cus, c->forced_splits);
+}
+
+static int kv_append_dev(Ctx *c, FullLayer *f, const float *k, const float *v, int64_t rows) {
+    if ((int64_t)f->len + rows > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %lld > capacity %d", f->len,
+                    (long long)rows, c->cfg.kv_capacity);
+    MFA_TRY(launch_kv_scatter(c->stream, c->cfg.kv_dtype, 0, c->cfg.num_kv_heads, c->cfg.head_dim,
+                              c->plane_elems, f->len, rows, k, v, f->k, f->v));
+    f->len += (int32_t)rows;
+    return MFA_OK;
+}
+
+static int gdn_step_dev(Ctx *c, LinearLayer *l, const float *qkv, const float *z,
+                        const float *alpha, const float *beta, float *out) {
+    if (!l->w.set) return fail(MFA_ERR_INVALID, "linear layer weights not set (mfa_set_linear_weights)");
+    MFA_TRY(launch_gdn_step(c->stream, c->cfg.linear_num_k_heads, c->cfg.linear_num_v_heads,
+                            c->cfg.linear_key_dim, c->cfg.linear_value_dim, c->cfg.conv_kernel_size,
+                            c->cfg.rms_norm_eps, l->w, l->conv_ring, l->step, l->ssm, qkv, z, alpha,
+                            beta, out));
+    l->step++;
+    return MFA_OK;
+}
+
+// A scratch device allocation for the stateless hooks.
+struct DevBuf {
+    void *p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int alloc(size_t bytes) {
+        MFA_HIP(hipMalloc(&p, bytes ? bytes : 4));
+        return MFA_OK;
+    }
+    int upload(const void *src, size_t bytes) {
+        MFA_TRY(alloc(bytes));
+        MFA_HIP(hipMemcpy(p, src, bytes, hipMemcpyHostToDevice));
+        return MFA_OK;
+    }
+    int download(void *dst, size_t bytes) {
+        MFA_HIP(hipDeviceSynchronize());
+        MFA_HIP(hipMemcpy(dst, p, bytes, hipMemcpyDeviceToHost));
+        return MFA_OK;
+    }
+    template <typename T> T *as() { return reinterpret_cast<T *>(p); }
+};
+
+static int sdpa_stateless(int kv_dtype, int32_t kv_len, int32_t Hq, int32_t Hkv, int32_t D,
+                          const float *q, const float *gate, const void *k, const void *v,
+                          float *out) {
+    if (!q || !gate || !k || !v || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (kv_len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", kv_len);
+    if (Hq <= 0 || Hkv <= 0 || D <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (Hq % Hkv != 0) return fail(MFA_ERR_INVALID, "num_attn_heads %d %% num_kv_heads %d != 0", Hq, Hkv);
+    if (!sdpa_shape_supported(kv_dtype, D)) return fail(MFA_ERR_SHAPE, "head_dim %d not supported", D);
+    const size_t es = kv_dtype == MFA_KV_BF16 ? 2 : 4;
+    const int blk = kv_dtype == MFA_KV_BF16 ? 32 : 16;
+    const int64_t cap = ((int64_t)kv_len + blk - 1) / blk * blk;
+    const size_t plane = (size_t)cap * D;
+    const size_t qd = (size_t)Hq * D, rows = (size_t)kv_len * Hkv * D;
+    int ncu = 256;
+    {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        MFA_HIP(hipGetDevice(&dev));
+        MFA_HIP(hipGetDeviceProperties(&prop, dev));
+        if (prop.multiProcessorCount > 0) ncu = prop.multiProcessorCount;
+    }
+    DevBuf dq, dg, dout, kr, vr, kt, vt, po, pml;
+    MFA_TRY(dq.upload(q, qd * 4));
+    MFA_TRY(dg.upload(gate, qd * 4));
+    MFA_TRY(dout.alloc(qd * 4));
+    MFA_TRY(kr.upload(k, rows * es));
+    MFA_TRY(vr.upload(v, rows * es));
+    MFA_TRY(kt.alloc(plane * Hkv * es));
+    MFA_TRY(vt.alloc(plane * Hkv * es));
+    MFA_HIP(hipMemsetAsync(kt.p, 0, plane * Hkv * es, nullptr));
+    MFA_HIP(hipMemsetAsync(vt.p, 0, plane * Hkv * es, nullptr));
+    MFA_TRY(launch_kv_scatter(nullptr, kv_dtype, kv_dtype == MFA_KV_BF16, Hkv, D, plane, 0, kv_len,
+                              kr.p, vr.p, kt.p, vt.p));
+    const int splits = sdpa_pick_splits(kv_dtype, Hq, Hkv, D, kv_len, ncu, 0);
+    SdpaWorkspace ws;
+    ws.part_o_elems = sdpa_workspace_o_elems(Hq, Hkv, D, splits);
+    ws.part_ml_elems = sdpa_workspace_ml_elems(Hq, Hkv, splits);
+    MFA_TRY(po.alloc(ws.part_o_elems * 4));
+    MFA_TRY(pml.alloc(ws.part_ml_elems * 4));
+    ws.part_o = po.as<float>();
+    ws.part_ml = pml.as<float>();
+    MFA_TRY(launch_sdpa_decode(nullptr, kv_dtype, Hq, Hkv, D, kv_len, plane, kt.p, vt.p,
+                               dq.as<float>(), dg.as<float>(), dout.as<float>(), ws, ncu, 0));
+    return dout.download(out, qd * 4);
+}
+
+}  // namespace mfa
+
+using namespace mfa;
+
+extern "C" {
+
+mfa_ctx *mfa_ctx_create(const mfa_config *cfg) {
+    Ctx *c = nullptr;
+    const int rc = create(cfg, &c);
+    if (rc != MFA_OK) {
+        const std::string keep = g_last_error;
+        destroy(c);
+        g_last_error = keep;
+        return nullptr;
+    }
+    return reinterpret_cast<mfa_ctx *>(c);
+}
+
+void mfa_ctx_destroy(mfa_ctx *ctx) { destroy(as_ctx(ctx)); }
+
+const char *mfa_last_error_string(void) { return g_last_error.c_str(); }
+
+int mfa_sync(mfa_ctx *ctx) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+void *mfa_stream(mfa_ctx *ctx) { return ctx ? (void *)as_ctx(ctx)->stream : nullptr; }
+
+int mfa_set_linear_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *conv_w_bf16,
+                           const float *a_log, const uint16_t *dt_bias_bf16,
+                           const uint16_t *norm_w_bf16) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!conv_w_bf16 || !a_log || !dt_bias_bf16 || !norm_w_bf16)
+        return fail(MFA_ERR_INVALID, "NULL weight pointer");
+    const size_t C = (size_t)c->conv_dim(), K = (size_t)c->cfg.conv_kernel_size;
+    const int Hv = c->cfg.linear_num_v_heads;
+    MFA_TRY(h2d(c, l->w.conv_w, conv_w_bf16, C * K * 2));
+    MFA_TRY(h2d(c, l->w.a_log, a_log, Hv * sizeof(float)));
+    MFA_TRY(h2d(c, l->w.dt_bias, dt_bias_bf16, Hv * 2));
+    MFA_TRY(h2d(c, l->w.norm_w, norm_w_bf16, (size_t)c->cfg.linear_value_dim * 2));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    l->w.set = true;
+    return MFA_OK;
+}
+
+int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (num_splits < 0) return fail(MFA_ERR_INVALID, "num_splits must be >= 0");
+    c->forced_splits = num_splits;
+    return MFA_OK;
+}
+
+/* ---- full attention -------------------------------------------------------- */
+
+int mfa_kv_append_dev(mfa_ctx *ctx, int32_t layer, const float *k_dev, const float *v_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!k_dev || !v_dev) return fail(MFA_ERR_INVALID, "NULL k/v row");
+    return kv_append_dev(c, f, k_dev, v_dev, 1);
+}
+
+int mfa_kv_append(mfa_ctx *ctx, int32_t layer, const float *k, const float *v) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!k || !v) return fail(MFA_ERR_INVALID, "NULL k/v row");
+    if (f->len + 1 > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d at capacity %d", f->len, c->cfg.kv_capacity);
+    const size_t kvd = (size_t)c->kv_dim();
+    MFA_TRY(ensure_stage(c, 2 * kvd));
+    MFA_TRY(h2d(c, c->stage, k, kvd * 4));
+    MFA_TRY(h2d(c, c->stage + kvd, v, kvd * 4));
+    MFA_TRY(kv_append_dev(c, f, c->stage, c->stage + kvd, 1));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+int32_t mfa_kv_len(mfa_ctx *ctx, int32_t layer) {
+    FullLayer *f;
+    const int rc = full_layer(as_ctx(ctx), layer, &f);
+    return rc != MFA_OK ? rc : f->len;
+}
+
+int mfa_sdpa_decode_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev, const float *q_gate_dev,
+                        float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_dev || !q_gate_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    return sdpa_decode_dev(c, f, q_dev, q_gate_dev, out_dev);
+}
+
+int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_gate, float *out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q || !q_gate || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
+    const size_t qd = (size_t)c->q_dim();
+    MFA_TRY(ensure_stage(c, 3 * qd));
+    MFA_TRY(h2d(c, c->stage, q, qd * 4));
+    MFA_TRY(h2d(c, c->stage + qd, q_gate, qd * 4));
+    MFA_TRY(sdpa_decode_dev(c, f, c->stage, c->stage + qd, c->stage + 2 * qd));
+    return d2h_sync(c, out, c->stage + 2 * qd, qd * 4);
+}
+
+int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_dev,
+                         const float *q_gate_dev, const float *k_dev, const float *v_dev,
+                         float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_dev || !q_gate_dev || !k_dev || !v_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    if ((int64_t)f->len + T > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %d > capacity %d", f->len, T,
+                    c->cfg.kv_capacity);
+    const size_t qd = (size_t)c->q_dim(), kvd = (size_t)c->kv_dim();
+    for (int t = 0; t < T; t++) {
+        MFA_TRY(kv_append_dev(c, f, k_dev + t * kvd, v_dev + t * kvd, 1));
+        MFA_TRY(sdpa_decode_dev(c, f, q_dev + t * qd, q_gate_dev + t * qd, out_dev + t * qd));
+    }
+    return MFA_OK;
+}
+
+int mfa_prefill_attn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q, const float *q_gate,
+                     const float *k, const float *v, float *out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q || !q_gate || !k || !v || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    const size_t qd = (size_t)c->q_dim() * T, kvd = (size_t)c->kv_dim() * T;
+    MFA_TRY(ensure_stage(c, 3 * qd + 2 * kvd));
+    float *dq = c->stage, *dg = dq + qd, *dout = dg + qd, *dk = dout + qd, *dv = dk + kvd;
+    MFA_TRY(h2d(c, dq, q, qd * 4));
+    MFA_TRY(h2d(c, dg, q_gate, qd * 4));
+    MFA_TRY(h2d(c, dk, k, kvd * 4));
+    MFA_TRY(h2d(c, dv, v, kvd * 4));
+    MFA_TRY(mfa_prefill_attn_dev(ctx, layer, T, dq, dg, dk, dv, dout));
+    return d2h_sync(c, out, dout, qd * 4);
+}
+
+/* ---- gated delta net --------------------------------------------------------- */
+
+int mfa_gdn_step_dev(mfa_ctx *ctx, int32_t layer, const float *qkv_in_dev, const float *z_dev,
+                     const float *alpha_dev, const float *beta_dev, float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!qkv_in_dev || !z_dev || !alpha_dev || !beta_dev || !out_dev)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    return gdn_step_dev(c, l, qkv_in_dev, z_dev, alpha_dev, beta_dev, out_dev);
+}
+
+int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv_in_dev,
+                        const float *z_dev, const float *alpha_dev, const float *beta_dev,
+                        float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!qkv_in_dev || !z_dev || !alpha_dev || !beta_dev || !out_dev)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    const size_t C = (size_t)c->conv_dim(), tv = (size_t)c->v_total(), Hv = (size_t)c->cfg.linear_num_v_heads;
+    for (int t = 0; t < T; t++)
+        MFA_TRY(gdn_step_dev(c, l, qkv_in_dev + t * C, z_dev + t * tv, alpha_dev + t * Hv,
+                             beta_dev + t * Hv, out_dev + t * tv));
+    return MFA_OK;
+}
+
+int mfa_prefill_gdn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv_in, const float *z,
+                    const float *alpha, const float *beta, float *out) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!qkv_in || !z || !alpha || !beta || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    const size_t C = (size_t)c->conv_dim() * T, tv = (size_t)c->v_total() * T,
+                 Hv = (size_t)c->cfg.linear_num_v_heads * T;
+    MFA_TRY(ensure_stage(c, C + 2 * tv + 2 * Hv));
+    float *dx = c->stage, *dz = dx + C, *dout = dz + tv, *da = dout + tv, *db = da + Hv;
+    MFA_TRY(h2d(c, dx, qkv_in, C * 4));
+    MFA_TRY(h2d(c, dz, z, tv * 4));
+    MFA_TRY(h2d(c, da, alpha, Hv * 4));
+    MFA_TRY(h2d(c, db, beta, Hv * 4));
+    MFA_TRY(mfa_prefill_gdn_dev(ctx, layer, T, dx, dz, da, db, dout));
+    return d2h_sync(c, out, dout, tv * 4);
+}
+
+int mfa_gdn_step(mfa_ctx *ctx, int32_t layer, const float *qkv_in, const float *z,
+                 const float *alpha, const float *beta, float *out) {
+    return mfa_prefill_gdn(ctx, layer, 1, qkv_in, z, alpha, beta, out);
+}
+
+/* ---- whole-stack sweep -------------------------------------------------------- */
+
+int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gate, float *full_out,
+                        const float *lin_qkv, const float *lin_z, const float *lin_alpha,
+                        const float *lin_beta, float *lin_out) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (!c->full.empty() && (!full_q || !full_gate || !full_out))
+        return fail(MFA_ERR_INVALID, "NULL full-attention argument");
+    if (!c->lin.empty() && (!lin_qkv || !lin_z || !lin_alpha || !lin_beta || !lin_out))
+        return fail(MFA_ERR_INVALID, "NULL linear-attention argument");
+    const size_t qd = (size_t)c->q_dim(), C = (size_t)c->conv_dim(), tv = (size_t)c->v_total(),
+                 Hv = (size_t)c->cfg.linear_num_v_heads;
+    for (int i = 0; i < c->cfg.num_layers; i++) {
+        const size_t s = (size_t)c->slot[i];
+        if (c->kind[i] == 1)
+            MFA_TRY(sdpa_decode_dev(c, &c->full[s], full_q + s * qd, full_gate + s * qd, full_out + s * qd));
+        else
+            MFA_TRY(gdn_step_dev(c, &c->lin[s], lin_qkv + s * C, lin_z + s * tv, lin_alpha + s * Hv,
+                                 lin_beta + s * Hv, lin_out + s * tv));
+    }
+    return MFA_OK;
+}
+
+/* ---- state operations ----------------------------------------------------------- */
+
+int mfa_reset(mfa_ctx *ctx) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    for (auto &f : c->full) MFA_TRY(truncate_full(c, f, 0));
+    for (auto &l : c->lin) MFA_TRY(reset_linear(c, l));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+int mfa_truncate(mfa_ctx *ctx, int32_t p0, int32_t p1) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    const int32_t new_len = p0 < 0 ? 0 : p0;
+    for (auto &f : c->full) {
+        const int32_t end = (p1 < 0 || p1 > f.len) ? f.len : p1;
+        MFA_TRY(truncate_full(c, f, new_len < end ? new_len : end));
+    }
+    for (auto &l : c->lin) MFA_TRY(reset_linear(c, l));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+int32_t mfa_pos_max(mfa_ctx *ctx) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    int32_t m = -1;
+    for (auto &f : c->full) m = f.len > m ? f.len : m;
+    return m;
+}
+
+int mfa_kv_export(mfa_ctx *ctx, int32_t layer, int32_t max_rows, float *k_out, float *v_out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!k_out || !v_out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (max_rows < f->len) return fail(MFA_ERR_INVALID, "buffer holds %d rows, layer has %d", max_rows, f->len);
+    if (f->len == 0) return MFA_OK;
+    const size_t n = (size_t)f->len * c->kv_dim();
+    MFA_TRY(ensure_stage(c, 2 * n));
+    MFA_TRY(launch_kv_gather(c->stream, c->cfg.kv_dtype, c->cfg.num_kv_heads, c->cfg.head_dim,
+                             c->plane_elems, f->len, f->k, f->v, c->stage, c->stage + n));
+    MFA_HIP(hipMemcpyAsync(k_out, c->stage, n * 4, hipMemcpyDeviceToHost, c->stream));
+    return d2h_sync(c, v_out, c->stage + n, n * 4);
+}
+
+static int kv_import(Ctx *c, int32_t layer, int32_t len, const void *k, const void *v, int src_bf16) {
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (len < 0) return fail(MFA_ERR_INVALID, "negative length");
+    if (len > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv import of %d rows exceeds capacity %d", len, c->cfg.kv_capacity);
+    if (len > 0 && (!k || !v)) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (src_bf16 && c->cfg.kv_dtype != MFA_KV_BF16)
+        return fail(MFA_ERR_INVALID, "bf16 rows need a bf16 cache");
+    MFA_TRY(truncate_full(c, *f, 0));
+    if (len > 0) {
+        const size_t n = (size_t)len * c->kv_dim();
+        const size_t es = src_bf16 ? 2 : 4;
+        MFA_TRY(ensure_stage(c, 2 * n));
+        char *dk = (char *)c->stage, *dv = dk + n * es;
+        MFA_TRY(h2d(c, dk, k, n * es));
+        MFA_TRY(h2d(c, dv, v, n * es));
+        MFA_TRY(launch_kv_scatter(c->stream, c->cfg.kv_dtype, src_bf16, c->cfg.num_kv_heads,
+                                  c->cfg.head_dim, c->plane_elems, 0, len, dk, dv, f->k, f->v));
+    }
+    f->len = len;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+int mfa_kv_import(mfa_ctx *ctx, int32_t layer, int32_t len, const float *k, const float *v) {
+    return kv_import(as_ctx(ctx), layer, len, k, v, 0);
+}
+
+int mfa_kv_import_bf16(mfa_ctx *ctx, int32_t layer, int32_t len, const uint16_t *k,
+                       const uint16_t *v) {
+    return kv_import(as_ctx(ctx), layer, len, k, v, 1);
+}
+
+int mfa_linear_state_export(mfa_ctx *ctx, int32_t layer, float *conv_state_out, float *ssm_state_out) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!conv_state_out || !ssm_state_out) return fail(MFA_ERR_INVALID, "NULL argument");
+    const int C = c->conv_dim(), K = c->cfg.conv_kernel_size;
+    const size_t nconv = (size_t)(K - 1) * C;
+    const size_t nssm = (size_t)c->cfg.linear_num_v_heads * c->cfg.linear_value_dim * c->cfg.linear_key_dim;
+    MFA_TRY(ensure_stage(c, nconv));
+    MFA_TRY(launch_conv_ring_export(c->stream, C, K, l->step, l->conv_ring, c->stage));
+    MFA_HIP(hipMemcpyAsync(conv_state_out, c->stage, nconv * 4, hipMemcpyDeviceToHost, c->stream));
+    return d2h_sync(c, ssm_state_out, l->ssm, nssm * 4);
+}
+
+int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state,
+                            const float *ssm_state) {
+    Ctx *c = as_ctx(ctx);
+    LinearLayer *l;
+    MFA_TRY(linear_layer(c, layer, &l));
+    if (!conv_state || !ssm_state) return fail(MFA_ERR_INVALID, "NULL argument");
+    const int C = c->conv_dim(), K = c->cfg.conv_kernel_size;
+    const size_t nconv = (size_t)(K - 1) * C;
+    const size_t nssm = (size_t)c->cfg.linear_num_v_heads * c->cfg.linear_value_dim * c->cfg.linear_key_dim;
+    MFA_TRY(ensure_stage(c, nconv));
+    MFA_TRY(h2d(c, c->stage, conv_state, nconv * 4));
+    MFA_TRY(launch_conv_ring_import(c->stream, C, K, c->stage, l->conv_ring));
+    MFA_TRY(h2d(c, l->ssm, ssm_state, nssm * 4));
+    l->step = 0;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
+}
+
+/* ---- timing ------------------------------------------------------------------------ */
+
+int mfa_timer_start(mfa_ctx *ctx) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    MFA_HIP(hipEventRecord(c->ev0, c->stream));
+    return MFA_OK;
+}
+
+int mfa_timer_stop(mfa_ctx *ctx, float *elapsed_ms) {
+    Ctx *c = as_ctx(ctx);
+    if (!c || !elapsed_ms) return fail(MFA_ERR_INVALID, "NULL argument");
+    MFA_HIP(hipEventRecord(c->ev1, c->stream));
+    MFA_HIP(hipEventSynchronize(c->ev1));
+    MFA_HIP(hipEventElapsedTime(elapsed_ms, c->ev0, c->ev1));
+    return MFA_OK;
+}
+
+/* ---- stateless hooks ------------------------------------------------------------------ */
+
+int mfa_sdpa(int32_t kv_len, int32_t Hq, int32_t Hkv, int32_t D, const float *q,
+             const float *q_gate, const float *k_cache, const float *v_cache, float *out) {
+    return sdpa_stateless(MFA_KV_F32, kv_len, Hq, Hkv, D, q, q_gate, k_cache, v_cache, out);
+}
+
+int mfa_sdpa_bf16kv(int32_t kv_len, int32_t Hq, int32_t Hkv, int32_t D, const float *q,
+                    const float *q_gate, const uint16_t *k_cache, const uint16_t *v_cache,
+                    float *out) {
+    return sdpa_stateless(MFA_KV_BF16, kv_len, Hq, Hkv, D, q, q_gate, k_cache, v_cache, out);
+}
+
+int mfa_attn_scores_batched(int32_t Hq, int32_t Hkv, int32_t D, int32_t L, const float *q,
+                            const float *k_cache, float scale, float *scores_out) {
+    if (!q || !k_cache || !scores_out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (Hq <= 0 || Hkv <= 0 || D <= 0 || L <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (Hq % Hkv != 0) return fail(MFA_ERR_INVALID, "num_heads %d %% num_kv_heads %d != 0", Hq, Hkv);
+    DevBuf dq, dk, ds;
+    MFA_TRY(dq.upload(q, (size_t)Hq * D * 4));
+    MFA_TRY(dk.upload(k_cache, (size_t)L * Hkv * D * 4));
+    MFA_TRY(ds.alloc((size_t)Hq * L * 4));
+    MFA_TRY(launch_attn_scores(nullptr, Hq, Hkv, D, L, L, dq.as<float>(), dk.as<float>(), scale, ds.as<float>()));
+    return ds.download(scores_out, (size_t)Hq * L * 4);
+}
+
+int mfa_attn_softmax_batched(int32_t Hq, int32_t L, float *scores_inout) {
+    if (!scores_inout) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (Hq <= 0 || L <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    DevBuf ds;
+    MFA_TRY(ds.upload(scores_inout, (size_t)Hq * L * 4));
+    MFA_TRY(launch_attn_softmax(nullptr, Hq, L, L, ds.as<float>()));
+    return ds.download(scores_inout, (size_t)Hq * L * 4);
+}
+
+int mfa_attn_values_batched(int32_t Hq, int32_t Hkv, int32_t D, int32_t L, const float *scores,
+                            const float *v_cache, float *out) {
+    if (!scores || !v_cache || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (Hq <= 0 || Hkv <= 0 || D <= 0 || L <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (Hq % Hkv != 0) return fail(MFA_ERR_INVALID, "num_heads %d %% num_kv_heads %d != 0", Hq, Hkv);
+    DevBuf ds, dv, dout;
+    MFA_TRY(ds.upload(scores, (size_t)Hq * L * 4));
+    MFA_TRY(dv.upload(v_cache, (size_t)L * Hkv * D * 4));
+    MFA_TRY(dout.alloc((size_t)Hq * D * 4));
+    MFA_TRY(launch_attn_values(nullptr, Hq, Hkv, D, L, L, ds.as<float>(), dv.as<float>(), dout.as<float>()));
+    return dout.download(out, (size_t)Hq * D * 4);
+}
+
+int mfa_sigmoid_gate(int32_t dim, const float *gate, float *x_inout) {
+    if (!gate || !x_inout) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (dim <= 0) return fail(MFA_ERR_INVALID, "non-positive dim");
+    DevBuf dg, dx;
+    MFA_TRY(dg.upload(gate, (size_t)dim * 4));
+    MFA_TRY(dx.upload(x_inout, (size_t)dim * 4));
+    MFA_TRY(launch_sigmoid_gate(nullptr, dim, dg.as<float>(), dx.as<float>()));
+    return dx.download(x_inout, (size_t)dim * 4);
+}
+
+int mfa_conv1d_step(int32_t C, int32_t K, float *conv_state_inout, const float *new_input,
+                    const uint16_t *weight_bf16, float *out) {
+    if (!conv_state_inout || !new_input || !weight_bf16 || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (C <= 0 || K < 2) return fail(MFA_ERR_INVALID, "bad conv shape: channels=%d kernel_size=%d", C, K);
+    DevBuf ds, di, dw, dout;
+    MFA_TRY(ds.upload(conv_state_inout, (size_t)(K - 1) * C * 4));
+    MFA_TRY(di.upload(new_input, (size_t)C * 4));
+    MFA_TRY(dw.upload(weight_bf16, (size_t)C * K * 2));
+    MFA_TRY(dout.alloc((size_t)C * 4));
+    MFA_TRY(launch_conv1d_step(nullptr, C, K, ds.as<float>(), di.as<float>(), dw.as<uint16_t>(), dout.as<float>()));
+    MFA_TRY(dout.download(out, (size_t)C * 4));
+    return ds.download(conv_state_inout, (size_t)(K - 1) * C * 4);
+}
+
+int mfa_rms_norm_qk(int32_t Hk, int32_t dk, float *q_inout, float *k_inout) {
+    if (!q_inout || !k_inout) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (Hk <= 0 || dk <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    DevBuf dq, dkb;
+    MFA_TRY(dq.upload(q_inout, (size_t)Hk * dk * 4));
+    MFA_TRY(dkb.upload(k_inout, (size_t)Hk * dk * 4));
+    MFA_TRY(launch_rms_norm_qk(nullptr, Hk, dk, dq.as<float>(), dkb.as<float>()));
+    MFA_TRY(dq.download(q_inout, (size_t)Hk * dk * 4));
+    return dkb.download(k_inout, (size_t)Hk * dk * 4);
+}
+
+int mfa_rms_norm_bare(int32_t dim, float eps, const float *x, float *out) {
+    if (!x || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (dim <= 0) return fail(MFA_ERR_INVALID, "dim must be positive");
+    DevBuf dx, dout;
+    MFA_TRY(dx.upload(x, (size_t)dim * 4));
+    MFA_TRY(dout.alloc((size_t)dim * 4));
+    MFA_TRY(launch_rms_norm_bare(nullptr, dim, eps, dx.as<float>(), dout.as<float>()));
+    return dout.download(out, (size_t)dim * 4);
+}
+
+int mfa_compute_decay_beta(int32_t Hv, const float *alpha, const float *beta, const float *a_log,
+                           const uint16_t *dt_bias_bf16, float *g_decay_out, float *beta_gate_out) {
+    if (!alpha || !beta || !a_log || !dt_bias_bf16 || !g_decay_out || !beta_gate_out)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    if (Hv <= 0) return fail(MFA_ERR_INVALID, "non-positive head count");
+    DevBuf da, db, dl, dt, dg, dbo;
+    MFA_TRY(da.upload(alpha, (size_t)Hv * 4));
+    MFA_TRY(db.upload(beta, (size_t)Hv * 4));
+    MFA_TRY(dl.upload(a_log, (size_t)Hv * 4));
+    MFA_TRY(dt.upload(dt_bias_bf16, (size_t)Hv * 2));
+    MFA_TRY(dg.alloc((size_t)Hv * 4));
+    MFA_TRY(dbo.alloc((size_t)Hv * 4));
+    MFA_TRY(launch_decay_beta(nullptr, Hv, da.as<float>(), db.as<float>(), dl.as<float>(),
+                              dt.as<uint16_t>(), dg.as<float>(), dbo.as<float>()));
+    MFA_TRY(dg.download(g_decay_out, (size_t)Hv * 4));
+    return dbo.download(beta_gate_out, (size_t)Hv * 4);
+}
+
+static int check_delta_shape(int32_t v_heads, int32_t k_heads, int32_t key_dim, int32_t value_dim) {
+    if (v_heads <= 0 || k_heads <= 0 || key_dim <= 0 || value_dim <= 0)
+        return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (v_heads % k_heads != 0)
+        return fail(MFA_ERR_INVALID, "v_heads %d is not a multiple of k_heads %d", v_heads, k_heads);
+    return MFA_OK;
+}
+
+int mfa_gated_delta_net_step(int32_t v_heads, int32_t k_heads, int32_t key_dim, int32_t value_dim,
+                             const float *g_decay, const float *beta_gate, const float *q,
+                             const float *k, const float *v, float *ssm_state_inout,
+                             float *out_values) {
+    if (!g_decay || !beta_gate || !q || !k || !v || !ssm_state_inout || !out_values)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    MFA_TRY(check_delta_shape(v_heads, k_heads, key_dim, value_dim));
+    const size_t nk = (size_t)k_heads * key_dim, nv = (size_t)v_heads * value_dim,
+                 ns = nv * key_dim;
+    DevBuf dg, db, dq, dk, dv, ds, dout;
+    MFA_TRY(dg.upload(g_decay, (size_t)v_heads * 4));
+    MFA_TRY(db.upload(beta_gate, (size_t)v_heads * 4));
+    MFA_TRY(dq.upload(q, nk * 4));
+    MFA_TRY(dk.upload(k, nk * 4));
+    MFA_TRY(dv.upload(v, nv * 4));
+    MFA_TRY(ds.upload(ssm_state_inout, ns * 4));
+    MFA_TRY(dout.alloc(nv * 4));
+    MFA_TRY(launch_delta_net_step(nullptr, v_heads, k_heads, key_dim, value_dim, dg.as<float>(),
+                                  db.as<float>(), dq.as<float>(), dk.as<float>(), dv.as<float>(),
+                                  ds.as<float>(), dout.as<float>()));
+    MFA_TRY(dout.download(out_values, nv * 4));
+    return ds.download(ssm_state_inout, ns * 4);
+}
+
+int mfa_gated_delta_recurrence(const float *a_log, const uint16_t *dt_bias_bf16, const float *alpha,
+                               const float *beta, const float *q, const float *k, const float *v,
+                               int32_t v_heads, int32_t k_heads, int32_t key_dim, int32_t value_dim,
+                               float *ssm_state_inout, float *out_values) {
+    if (!a_log || !dt_bias_bf16 || !alpha || !beta || !q || !k || !v || !ssm_state_inout || !out_values)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    MFA_TRY(check_delta_shape(v_heads, k_heads, key_dim, value_dim));
+    const size_t nk = (size_t)k_heads * key_dim, nv = (size_t)v_heads * value_dim,
+                 ns = nv * key_dim;
+    DevBuf da, db, dl, dt, dg, dbo, dq, dk, dv, ds, dout;
+    MFA_TRY(da.upload(alpha, (size_t)v_heads * 4));
+    MFA_TRY(db.upload(beta, (size_t)v_heads * 4));
+    MFA_TRY(dl.upload(a_log, (size_t)v_heads * 4));
+    MFA_TRY(dt.upload(dt_bias_bf16, (size_t)v_heads * 2));
+    MFA_TRY(dg.alloc((size_t)v_heads * 4));
+    MFA_TRY(dbo.alloc((size_t)v_heads * 4));
+    MFA_TRY(dq.upload(q, nk * 4));
+    MFA_TRY(dk.upload(k, nk * 4));
+    MFA_TRY(dv.upload(v, nv * 4));
+    MFA_TRY(ds.upload(ssm_state_inout, ns * 4));
+    MFA_TRY(dout.alloc(nv * 4));
+    MFA_TRY(launch_decay_beta(nullptr, v_heads, da.as<float>(), db.as<float>(), dl.as<float>(),
+                              dt.as<uint16_t>(), dg.as<float>(), dbo.as<float>()));
+    MFA_TRY(launch_delta_net_step(nullptr, v_heads, k_heads, key_dim, value_dim, dg.as<float>(),
+                                  dbo.as<float>(), dq.as<float>(), dk.as<float>(), dv.as<float>(),
+                                  ds.as<float>(), dout.as<float>()));
+    MFA_TRY(dout.download(out_values, nv * 4));
+    return ds.download(ssm_state_inout, ns * 4);
+}
+
+int mfa_gated_rms_norm(int32_t H, int32_t dim, float eps, const float *x, const float *z,
+                       const uint16_t *weight_bf16, float *out) {
+    if (!x || !z || !weight_bf16 || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (H <= 0 || dim <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    const size_t n = (size_t)H * dim;
+    DevBuf dx, dz, dw, dout;
+    MFA_TRY(dx.upload(x, n * 4));
+    MFA_TRY(dz.upload(z, n * 4));
+    MFA_TRY(dw.upload(weight_bf16, (size_t)dim * 2));
+    MFA_TRY(dout.alloc(n * 4));
+    MFA_TRY(launch_gated_rms_norm(nullptr, H, dim, eps, dx.as<float>(), dz.as<float>(),
+                                  dw.as<uint16_t>(), dout.as<float>()));
+    return dout.download(out, n * 4);
+}
+
+}  // extern "C"

@@ -1,0 +1,219 @@
+// Internal declarations shared by the translation units of libmoeflux_attn_hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "moeflux_attn.h"
+
+namespace mfa {
+
+// ---- error plumbing --------------------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+
+#define MFA_HIP(expr)                                                                  \
+    do {                                                                               \
+        hipError_t _e = (expr);                                                        \
+        if (_e != hipSuccess)                                                          \
+            return ::mfa::fail(MFA_ERR_HIP, "%s failed: %s (%s:%d)", #expr,            \
+                               hipGetErrorString(_e), __FILE__, __LINE__);             \
+    } while (0)
+
+#define MFA_TRY(expr)              \
+    do {                           \
+        int _rc = (expr);          \
+        if (_rc != MFA_OK) return _rc; \
+    } while (0)
+
+// ---- small device helpers ---------------------------------------------------
+__host__ __device__ inline float bf16_bits_to_f32(uint16_t b) {
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)b) << 16;
+    return c.f;
+}
+
+// round-to-nearest-even; NaN stays NaN.
+__host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    uint32_t u = c.u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// ---- KV cache tiling ---------------------------------------------------------
+// The device KV cache is stored in the order the decode kernel's MFMA operands
+// consume it, so that every wave-level load is one contiguous 1 KiB run and
+// goes straight from HBM into matrix-core operand registers.
+//
+// One plane per (layer, K|V, kv head).  Positions are grouped in blocks
+// (32 positions for bf16, 16 for f32); a block of one plane is contiguous.
+//
+// bf16, block of 32 positions, element (p, x) with p in [0,32), x in [0,D):
+//   K: [sub = p/16][chunk = x/8][row = p%16][e = x%8]
+//   V: [dt = x/16][g = (p%16)/4][m = x%16][e = 4*(p/16) + p%4]
+// f32, block of 16 positions:
+//   K: [chunk = x/4][row = p][e = x%4]
+//   V: [i = p%4][c = x/64][g = p/4][m = (x%64)/4][j = x%4]
+template <typename T> struct KvTile;
+
+template <> struct KvTile<uint16_t> {
+    static constexpr int BLK = 32;
+    __host__ __device__ static inline int64_t k_off(int64_t pos, int x, int D) {
+        const int64_t blk = pos / 32;
+        const int p = (int)(pos % 32);
+        return blk * 32 * D + ((int64_t)(p / 16) * (D / 8) + x / 8) * 128 + (p % 16) * 8 + (x % 8);
+    }
+    __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
+        const int64_t blk = pos / 32;
+        const int p = (int)(pos % 32);
+        const int g = (p % 16) / 4;
+        const int e = 4 * (p / 16) + (p % 4);
+        return blk * 32 * D + (((int64_t)(x / 16) * 4 + g) * 16 + (x % 16)) * 8 + e;
+    }
+};
+
+template <> struct KvTile<float> {
+    static constexpr int BLK = 16;
+    __host__ __device__ static inline int64_t k_off(int64_t pos, int x, int D) {
+        const int64_t blk = pos / 16;
+        const int p = (int)(pos % 16);
+        return blk * 16 * D + ((int64_t)(x / 4) * 16 + p) * 4 + (x % 4);
+    }
+    __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
+        const int64_t blk = pos / 16;
+        const int p = (int)(pos % 16);
+        const int i = p % 4, g = p / 4;
+        const int c = x / 64, m = (x % 64) / 4, j = x % 4;
+        return blk * 16 * D + ((((int64_t)i * (D / 64) + c) * 4 + g) * 16 + m) * 4 + j;
+    }
+};
+
+// ---- context ----------------------------------------------------------------
+struct LinearWeights {
+    uint16_t *conv_w = nullptr;  // [C, K] bf16
+    float *a_log = nullptr;      // [Hv]
+    uint16_t *dt_bias = nullptr; // [Hv] bf16
+    uint16_t *norm_w = nullptr;  // [dv] bf16
+    bool set = false;
+};
+
+struct FullLayer {
+    void *k = nullptr;  // [Hkv] planes, tiled (see KvTile)
+    void *v = nullptr;
+    int32_t len = 0;
+};
+
+struct LinearLayer {
+    float *conv_ring = nullptr; // [K, C] ring of the last K inputs (slot = step % K)
+    float *ssm = nullptr;       // [Hv, dv, dk]
+    int64_t step = 0;           // tokens consumed since the last reset/import
+    LinearWeights w;
+};
+
+struct Ctx {
+    mfa_config cfg{};
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::vector<int> kind;      // per layer: 1 = full attention, 0 = linear
+    std::vector<int> slot;      // index into full / lin
+    std::vector<FullLayer> full;
+    std::vector<LinearLayer> lin;
+    int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
+    size_t plane_elems = 0;     // elements of one (layer, K|V, kv head) plane
+    // split-K workspace
+    float *part_o = nullptr;
+    float *part_ml = nullptr;
+    size_t part_o_elems = 0, part_ml_elems = 0;
+    int32_t forced_splits = 0;
+    // host-pointer staging
+    float *stage = nullptr;
+    size_t stage_elems = 0;
+    float *pinned = nullptr;
+    size_t pinned_elems = 0;
+    int num_cus = 256;
+
+    int conv_dim() const {
+        return 2 * cfg.linear_num_k_heads * cfg.linear_key_dim +
+               cfg.linear_num_v_heads * cfg.linear_value_dim;
+    }
+    int q_dim() const { return cfg.num_attn_heads * cfg.head_dim; }
+    int kv_dim() const { return cfg.num_kv_heads * cfg.head_dim; }
+    int v_total() const { return cfg.linear_num_v_heads * cfg.linear_value_dim; }
+    size_t kv_elem_size() const { return cfg.kv_dtype == MFA_KV_BF16 ? 2 : 4; }
+};
+
+inline Ctx *as_ctx(mfa_ctx *c) { return reinterpret_cast<Ctx *>(c); }
+
+int full_layer(Ctx *c, int32_t layer, FullLayer **out);
+int linear_layer(Ctx *c, int32_t layer, LinearLayer **out);
+int ensure_stage(Ctx *c, size_t elems);
+
+// ---- kernel launchers (device pointers, asynchronous on `stream`) ------------
+
+// sdpa_decode.hip
+struct SdpaWorkspace {
+    float *part_o;
+    float *part_ml;
+    size_t part_o_elems, part_ml_elems;
+};
+bool sdpa_shape_supported(int kv_dtype, int head_dim);
+// Number of splits the launcher will use (for workspace sizing pass kv_len = capacity).
+int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced);
+size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits);
+size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits);
+int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
+                       size_t plane_elems, const void *k_tiled, const void *v_tiled,
+                       const float *q, const float *gate, float *out, const SdpaWorkspace &ws,
+                       int num_cus, int forced_splits);
+// Scatter `n_rows` row-major rows ([n_rows, Hkv*D], f32 or bf16 source) into the
+// tiled planes starting at position pos0.
+int launch_kv_scatter(hipStream_t stream, int kv_dtype, int src_is_bf16, int Hkv, int D,
+                      size_t plane_elems, int64_t pos0, int64_t n_rows, const void *k_rows,
+                      const void *v_rows, void *k_tiled, void *v_tiled);
+// Gather positions [0, n_rows) back to row-major f32.
+int launch_kv_gather(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plane_elems,
+                     int64_t n_rows, const void *k_tiled, const void *v_tiled, float *k_rows,
+                     float *v_rows);
+// Zero positions [pos0, pos1) of every plane.
+int launch_kv_zero(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plane_elems,
+                   int64_t pos0, int64_t pos1, void *k_tiled, void *v_tiled);
+
+// attn_kernels.hip (the four reference kernels, one launch each)
+int launch_attn_scores(hipStream_t s, int Hq, int Hkv, int D, int L, int stride, const float *q,
+                       const float *k, float scale, float *scores);
+int launch_attn_softmax(hipStream_t s, int Hq, int L, int stride, float *scores);
+int launch_attn_values(hipStream_t s, int Hq, int Hkv, int D, int L, int stride,
+                       const float *scores, const float *v, float *out);
+int launch_sigmoid_gate(hipStream_t s, int dim, const float *gate, float *x);
+
+// gdn.hip
+bool gdn_shape_supported(int Hk, int Hv, int dk, int dv, int K);
+int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps,
+                    const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
+                    const float *qkv_in, const float *z, const float *alpha, const float *beta,
+                    float *out);
+int launch_conv1d_step(hipStream_t s, int C, int K, float *conv_state, const float *in,
+                       const uint16_t *w, float *out);
+int launch_rms_norm_qk(hipStream_t s, int Hk, int dk, float *q, float *k);
+int launch_rms_norm_bare(hipStream_t s, int dim, float eps, const float *x, float *out);
+int launch_decay_beta(hipStream_t s, int Hv, const float *alpha, const float *beta,
+                      const float *a_log, const uint16_t *dt_bias, float *g, float *b);
+int launch_delta_net_step(hipStream_t s, int Hv, int Hk, int dk, int dv, const float *g,
+                          const float *b, const float *q, const float *k, const float *v,
+                          float *ssm, float *out);
+int launch_gated_rms_norm(hipStream_t s, int H, int dim, float eps, const float *x,
+                          const float *z, const uint16_t *w, float *out);
+// ring <-> time-major conversion of the conv state
+int launch_conv_ring_export(hipStream_t s, int C, int K, int64_t step, const float *ring,
+                            float *state_out);
+int launch_conv_ring_import(hipStream_t s, int C, int K, const float *state, float *ring);
+
+}  // namespace mfa

@@ -1,0 +1,462 @@
+/*
+ * CPU oracle for the per-token attention path (gated GQA SDPA decode and the
+ * Gated-DeltaNet step).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP kernels are
+ * compared against and the code timed as the CPU baseline.  Nothing in the
+ * shipped library links, loads or calls it.
+ *
+ * Every function is a plain scalar fp32 restatement, written from the text of
+ * the reference (no reference source is compiled or copied); the citation
+ * above each function names the lines it follows.  Built with
+ * -ffp-contract=off so that a*b+c is two roundings exactly where the Rust
+ * reference writes `a * b + c`, and fmaf() is used exactly where the Rust
+ * reference writes `mul_add`.
+ *
+ * Pinning status (which independent check holds each function in place is
+ * listed in tests/test_oracle_pinning.py):
+ *   orc_sdpa, orc_sdpa_bf16kv, orc_attn_scores, orc_attn_softmax,
+ *   orc_attn_values, orc_sigmoid_gate, orc_conv1d_step, orc_conv_state_shift,
+ *   orc_rms_norm_bare, orc_rms_norm_qk, orc_rms_norm_gated, orc_decay_beta,
+ *   orc_gated_delta_recurrence, orc_gdn_step, orc_prefill_attn,
+ *   orc_prefill_gdn : pinned by float64 brute force on small shapes, closed
+ *   forms and invariants (the reference holds no numeric vectors for them).
+ *   The Accelerate-BLAS variant of the recurrence (infer.m:4954-4993) is not
+ *   restated: parity unpinned at that boundary (mathematically identical to
+ *   orc_gated_delta_recurrence).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* crates/moeflux/src/riir/embedding.rs:153-155 — bf16 is the top half of an f32. */
+static inline float orc_bf16_to_f32(uint16_t bits) {
+    uint32_t u = ((uint32_t)bits) << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* Round-to-nearest-even f32 -> bf16.  Used only to make test inputs; both the
+ * oracle and the HIP path are fed the identical bits, so the rounding mode
+ * never enters a parity comparison. */
+ORC_API uint16_t orc_f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+ORC_API void orc_f32_to_bf16_array(const float *x, uint16_t *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = orc_f32_to_bf16(x[i]);
+}
+
+ORC_API void orc_bf16_to_f32_array(const uint16_t *x, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = orc_bf16_to_f32(x[i]);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Full attention                                                           */
+/* ------------------------------------------------------------------------ */
+
+/* crates/moeflux/src/riir/sdpa.rs:63-172 (C twin infer.m:762-804, softmax
+ * infer.m:821-835).  Per head: s[p] = (q_h . K[p,kv_h]) * scale, softmax with
+ * the max taken from s[0], expf, multiply by 1/sum; o_h = sum_p w[p] V[p,kv_h];
+ * then out *= 1/(1+expf(-gate)).  Returns -1 on the argument errors the
+ * reference rejects (sdpa.rs:71, moeflux.h:177-178). */
+ORC_API int orc_sdpa(int32_t kv_len, int32_t num_attn_heads, int32_t num_kv_heads,
+                     int32_t head_dim, const float *q, const float *q_gate,
+                     const float *k_cache, const float *v_cache, float *out) {
+    if (!q || !q_gate || !k_cache || !v_cache || !out) return -1;
+    if (kv_len <= 0 || num_attn_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0) return -1;
+    if (num_attn_heads % num_kv_heads != 0) return -1;
+    const int q_dim = num_attn_heads * head_dim;
+    const int64_t kv_dim = (int64_t)num_kv_heads * head_dim;
+    const int heads_per_kv = num_attn_heads / num_kv_heads;
+    const float scale = 1.0f / sqrtf((float)head_dim);
+
+    for (int i = 0; i < q_dim; i++) out[i] = 0.0f;
+    float *scores = (float *)malloc((size_t)kv_len * sizeof(float));
+    if (!scores) return -1;
+    for (int h = 0; h < num_attn_heads; h++) {
+        const int kv_h = h / heads_per_kv;
+        const float *qh = q + (int64_t)h * head_dim;
+        for (int p = 0; p < kv_len; p++) {
+            const float *kp = k_cache + (int64_t)p * kv_dim + (int64_t)kv_h * head_dim;
+            float dot = 0.0f;
+            for (int d = 0; d < head_dim; d++) dot += qh[d] * kp[d];
+            scores[p] = dot * scale;
+        }
+        float max_val = scores[0];
+        for (int p = 1; p < kv_len; p++)
+            if (scores[p] > max_val) max_val = scores[p];
+        float sum = 0.0f;
+        for (int p = 0; p < kv_len; p++) {
+            scores[p] = expf(scores[p] - max_val);
+            sum += scores[p];
+        }
+        const float inv_sum = 1.0f / sum;
+        for (int p = 0; p < kv_len; p++) scores[p] *= inv_sum;
+
+        float *oh = out + (int64_t)h * head_dim;
+        for (int p = 0; p < kv_len; p++) {
+            const float *vp = v_cache + (int64_t)p * kv_dim + (int64_t)kv_h * head_dim;
+            const float w = scores[p];
+            for (int d = 0; d < head_dim; d++) oh[d] += w * vp[d];
+        }
+    }
+    free(scores);
+    for (int i = 0; i < q_dim; i++) {
+        const float g = 1.0f / (1.0f + expf(-q_gate[i]));
+        out[i] *= g;
+    }
+    return 0;
+}
+
+/* The same function over a bf16 K/V cache: the stored bits are widened exactly
+ * (embedding.rs:153-155) and everything else is orc_sdpa.  The reference has no
+ * bf16 cache; its semantics are defined as sdpa.rs:63-172 on the widened
+ * values. */
+ORC_API int orc_sdpa_bf16kv(int32_t kv_len, int32_t num_attn_heads, int32_t num_kv_heads,
+                            int32_t head_dim, const float *q, const float *q_gate,
+                            const uint16_t *k_cache, const uint16_t *v_cache, float *out) {
+    if (!k_cache || !v_cache) return -1;
+    if (kv_len <= 0 || num_kv_heads <= 0 || head_dim <= 0) return -1;
+    const int64_t n = (int64_t)kv_len * num_kv_heads * head_dim;
+    float *kf = (float *)malloc((size_t)n * sizeof(float));
+    float *vf = (float *)malloc((size_t)n * sizeof(float));
+    if (!kf || !vf) { free(kf); free(vf); return -1; }
+    for (int64_t i = 0; i < n; i++) { kf[i] = orc_bf16_to_f32(k_cache[i]); vf[i] = orc_bf16_to_f32(v_cache[i]); }
+    int rc = orc_sdpa(kv_len, num_attn_heads, num_kv_heads, head_dim, q, q_gate, kf, vf, out);
+    free(kf); free(vf);
+    return rc;
+}
+
+/* crates/moeflux/shaders/shaders.metal:976-1019 (host contract moeflux.h:475-483):
+ * scores[h*seq_stride + p] = (Q[h] . K[p, h/heads_per_kv]) * scale. */
+ORC_API int orc_attn_scores(int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t seq_len, int32_t seq_stride, const float *q,
+                            const float *k_cache, float scale, float *scores_out) {
+    if (!q || !k_cache || !scores_out) return -1;
+    if (num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || seq_len <= 0) return -1;
+    if (num_heads % num_kv_heads != 0 || seq_stride < seq_len) return -1;
+    const int hpk = num_heads / num_kv_heads;
+    const int64_t kv_dim = (int64_t)num_kv_heads * head_dim;
+    for (int h = 0; h < num_heads; h++) {
+        const float *qh = q + (int64_t)h * head_dim;
+        for (int p = 0; p < seq_len; p++) {
+            const float *kp = k_cache + (int64_t)p * kv_dim + (int64_t)(h / hpk) * head_dim;
+            float acc = 0.0f;
+            for (int d = 0; d < head_dim; d++) acc += qh[d] * kp[d];
+            scores_out[(int64_t)h * seq_stride + p] = acc * scale;
+        }
+    }
+    return 0;
+}
+
+/* crates/moeflux/shaders/shaders.metal:1026-1084: per-head softmax in place;
+ * running max starts at -1e30f, exp, multiply by 1/sum. */
+ORC_API int orc_attn_softmax(int32_t num_heads, int32_t seq_len, int32_t seq_stride,
+                             float *scores) {
+    if (!scores || num_heads <= 0 || seq_len <= 0 || seq_stride < seq_len) return -1;
+    for (int h = 0; h < num_heads; h++) {
+        float *s = scores + (int64_t)h * seq_stride;
+        float m = -1e30f;
+        for (int i = 0; i < seq_len; i++) m = s[i] > m ? s[i] : m;
+        float sum = 0.0f;
+        for (int i = 0; i < seq_len; i++) { s[i] = expf(s[i] - m); sum += s[i]; }
+        const float inv = 1.0f / sum;
+        for (int i = 0; i < seq_len; i++) s[i] *= inv;
+    }
+    return 0;
+}
+
+/* crates/moeflux/shaders/shaders.metal:1095-1117:
+ * out[h,d] = sum_p scores[h*seq_stride+p] * V[p, kv_h*head_dim + d], p ascending. */
+ORC_API int orc_attn_values(int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t seq_len, int32_t seq_stride, const float *scores,
+                            const float *v_cache, float *out) {
+    if (!scores || !v_cache || !out) return -1;
+    if (num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || seq_len <= 0) return -1;
+    if (num_heads % num_kv_heads != 0 || seq_stride < seq_len) return -1;
+    const int hpk = num_heads / num_kv_heads;
+    const int64_t kv_dim = (int64_t)num_kv_heads * head_dim;
+    for (int h = 0; h < num_heads; h++) {
+        const float *s = scores + (int64_t)h * seq_stride;
+        for (int d = 0; d < head_dim; d++) {
+            float acc = 0.0f;
+            for (int p = 0; p < seq_len; p++)
+                acc += s[p] * v_cache[(int64_t)p * kv_dim + (int64_t)(h / hpk) * head_dim + d];
+            out[(int64_t)h * head_dim + d] = acc;
+        }
+    }
+    return 0;
+}
+
+/* crates/moeflux/shaders/shaders.metal:1125-1134: x[i] *= 1/(1+exp(-gate[i])). */
+ORC_API int orc_sigmoid_gate(int32_t dim, const float *gate, float *x_inout) {
+    if (!gate || !x_inout || dim <= 0) return -1;
+    for (int i = 0; i < dim; i++) {
+        const float g = 1.0f / (1.0f + expf(-gate[i]));
+        x_inout[i] = x_inout[i] * g;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Gated DeltaNet                                                           */
+/* ------------------------------------------------------------------------ */
+
+/* crates/moeflux/src/riir/linear_attn.rs:89-156 (C twin infer.m:922-945):
+ * acc = fma(state[k,c], w[c,k], acc) for k < K-1, then fma(in[c], w[c,K-1], acc);
+ * out = acc / (1 + exp(-acc)).  conv_state is [(K-1), channels] time-major, the
+ * weight is bf16 [channels, K] channel-major.  Does not advance the state. */
+ORC_API int orc_conv1d_step(const float *conv_state, const float *new_input,
+                            const uint16_t *weight_bf16, int32_t channels,
+                            int32_t kernel_size, float *out) {
+    if (!conv_state || !new_input || !weight_bf16 || !out) return -1;
+    if (channels <= 0 || kernel_size <= 0) return -1;
+    for (int c = 0; c < channels; c++) {
+        float acc = 0.0f;
+        for (int k = 0; k < kernel_size - 1; k++) {
+            const float w = orc_bf16_to_f32(weight_bf16[(int64_t)c * kernel_size + k]);
+            acc = fmaf(conv_state[(int64_t)k * channels + c], w, acc);
+        }
+        const float w = orc_bf16_to_f32(weight_bf16[(int64_t)c * kernel_size + (kernel_size - 1)]);
+        acc = fmaf(new_input[c], w, acc);
+        out[c] = acc;
+    }
+    for (int c = 0; c < channels; c++) out[c] = out[c] / (1.0f + expf(-out[c]));
+    return 0;
+}
+
+/* crates/moeflux-sys/metal_infer/infer.m:2636-2639 (= shaders.metal:1241-1243):
+ * drop the oldest slot, append the new input as the newest. */
+ORC_API int orc_conv_state_shift(float *conv_state, const float *new_input,
+                                 int32_t channels, int32_t kernel_size) {
+    if (!conv_state || !new_input || channels <= 0 || kernel_size < 2) return -1;
+    memmove(conv_state, conv_state + channels,
+            (size_t)(kernel_size - 2) * channels * sizeof(float));
+    memcpy(conv_state + (size_t)(kernel_size - 2) * channels, new_input,
+           (size_t)channels * sizeof(float));
+    return 0;
+}
+
+/* crates/moeflux/src/riir/linear_attn.rs:160-184: out = x / sqrt(mean(x^2)+eps). */
+ORC_API int orc_rms_norm_bare(int32_t dim, float eps, const float *x, float *out) {
+    if (!x || !out || dim <= 0) return -1;
+    float sum_sq = 0.0f;
+    for (int i = 0; i < dim; i++) sum_sq += x[i] * x[i];
+    const float inv_rms = 1.0f / sqrtf(sum_sq / (float)dim + eps);
+    for (int i = 0; i < dim; i++) out[i] = x[i] * inv_rms;
+    return 0;
+}
+
+/* crates/moeflux-sys/metal_infer/infer.m:2655-2667 (= shaders.metal:1254-1303):
+ * per k-head bare RMS norm with eps 1e-6, then q *= (1/sqrt(dk))^2 and
+ * k *= 1/sqrt(dk).  In place. */
+ORC_API int orc_rms_norm_qk(int32_t num_k_heads, int32_t key_dim, float *q, float *k) {
+    if (!q || !k || num_k_heads <= 0 || key_dim <= 0) return -1;
+    const float inv_scale = 1.0f / sqrtf((float)key_dim);
+    for (int h = 0; h < num_k_heads; h++) {
+        float *qh = q + (int64_t)h * key_dim;
+        orc_rms_norm_bare(key_dim, 1e-6f, qh, qh);
+        const float q_scale = inv_scale * inv_scale;
+        for (int d = 0; d < key_dim; d++) qh[d] *= q_scale;
+    }
+    for (int h = 0; h < num_k_heads; h++) {
+        float *kh = k + (int64_t)h * key_dim;
+        orc_rms_norm_bare(key_dim, 1e-6f, kh, kh);
+        for (int d = 0; d < key_dim; d++) kh[d] *= inv_scale;
+    }
+    return 0;
+}
+
+/* crates/moeflux/src/riir/linear_attn.rs:190-242 (C twin infer.m:2529-2539):
+ * out = x * inv_rms(x) * w * silu(z), left-to-right products. */
+ORC_API int orc_rms_norm_gated(int32_t dim, float eps, const float *x, const float *z,
+                               const uint16_t *w_bf16, float *out) {
+    if (!x || !z || !w_bf16 || !out || dim <= 0) return -1;
+    float sum_sq = 0.0f;
+    for (int i = 0; i < dim; i++) sum_sq += x[i] * x[i];
+    const float inv_rms = 1.0f / sqrtf(sum_sq / (float)dim + eps);
+    for (int i = 0; i < dim; i++) {
+        const float w = orc_bf16_to_f32(w_bf16[i]);
+        const float silu_z = z[i] / (1.0f + expf(-z[i]));
+        out[i] = x[i] * inv_rms * w * silu_z;
+    }
+    return 0;
+}
+
+/* crates/moeflux/src/riir/linear_attn.rs:357-370 (= shaders.metal:1312-1327):
+ * g = exp(-exp(A_log) * log(1 + exp(alpha + dt_bias))), beta_gate = sigmoid(beta).
+ * The softplus is the naive form and overflows to +inf (g = 0) for large
+ * arguments, as the reference's does. */
+ORC_API int orc_decay_beta(int32_t v_heads, const float *alpha, const float *beta,
+                           const float *a_log, const uint16_t *dt_bias_bf16,
+                           float *g_decay, float *beta_gate) {
+    if (!alpha || !beta || !a_log || !dt_bias_bf16 || !g_decay || !beta_gate) return -1;
+    if (v_heads <= 0) return -1;
+    for (int vh = 0; vh < v_heads; vh++) {
+        const float dt_b = orc_bf16_to_f32(dt_bias_bf16[vh]);
+        const float a_capital = expf(a_log[vh]);
+        const float softplus_val = logf(1.0f + expf(alpha[vh] + dt_b));
+        g_decay[vh] = expf(-a_capital * softplus_val);
+        beta_gate[vh] = 1.0f / (1.0f + expf(-beta[vh]));
+    }
+    return 0;
+}
+
+/* crates/moeflux/shaders/shaders.metal:1154-1194 — the recurrence proper with
+ * g and beta_gate already computed.  Loops follow linear_attn.rs:373-411: decay
+ * the whole head state; per row kv_mem via fma, delta = (v - kv_mem) * beta,
+ * S[vi,:] = fma(k, delta, S[vi,:]); then out[vi] = S[vi,:] . q via fma. */
+ORC_API int orc_delta_net_step(int32_t v_heads, int32_t k_heads, int32_t key_dim,
+                               int32_t value_dim, const float *g_decay,
+                               const float *beta_gate, const float *q, const float *k,
+                               const float *v, float *ssm_state, float *out_values) {
+    if (!g_decay || !beta_gate || !q || !k || !v || !ssm_state || !out_values) return -1;
+    if (v_heads <= 0 || k_heads <= 0 || key_dim <= 0 || value_dim <= 0) return -1;
+    if (v_heads % k_heads != 0) return -1;
+    const int k_heads_per_v = v_heads / k_heads;
+    const int64_t head_stride = (int64_t)value_dim * key_dim;
+    for (int vh = 0; vh < v_heads; vh++) {
+        const int kh = vh / k_heads_per_v;
+        const float g = g_decay[vh];
+        const float b_gate = beta_gate[vh];
+        float *S = ssm_state + (int64_t)vh * head_stride;
+        const float *kk = k + (int64_t)kh * key_dim;
+        const float *qq = q + (int64_t)kh * key_dim;
+        const float *vv = v + (int64_t)vh * value_dim;
+        float *oo = out_values + (int64_t)vh * value_dim;
+        for (int64_t i = 0; i < head_stride; i++) S[i] *= g;
+        for (int vi = 0; vi < value_dim; vi++) {
+            float *row = S + (int64_t)vi * key_dim;
+            float kv_mem = 0.0f;
+            for (int ki = 0; ki < key_dim; ki++) kv_mem = fmaf(row[ki], kk[ki], kv_mem);
+            const float delta = (vv[vi] - kv_mem) * b_gate;
+            for (int ki = 0; ki < key_dim; ki++) row[ki] = fmaf(kk[ki], delta, row[ki]);
+        }
+        for (int vi = 0; vi < value_dim; vi++) {
+            const float *row = S + (int64_t)vi * key_dim;
+            float sum = 0.0f;
+            for (int ki = 0; ki < key_dim; ki++) sum = fmaf(row[ki], qq[ki], sum);
+            oo[vi] = sum;
+        }
+    }
+    return 0;
+}
+
+/* crates/moeflux/src/riir/linear_attn.rs:288-414 (C twin infer.m:7931-7988):
+ * decay/beta precomputation followed by the recurrence. */
+ORC_API int orc_gated_delta_recurrence(const float *a_log, const uint16_t *dt_bias_bf16,
+                                       const float *alpha, const float *beta,
+                                       const float *q, const float *k, const float *v,
+                                       int32_t v_heads, int32_t k_heads, int32_t key_dim,
+                                       int32_t value_dim, float *ssm_state,
+                                       float *out_values) {
+    if (v_heads <= 0) return -1;
+    float *g = (float *)malloc((size_t)v_heads * sizeof(float));
+    float *b = (float *)malloc((size_t)v_heads * sizeof(float));
+    if (!g || !b) { free(g); free(b); return -1; }
+    int rc = orc_decay_beta(v_heads, alpha, beta, a_log, dt_bias_bf16, g, b);
+    if (rc == 0)
+        rc = orc_delta_net_step(v_heads, k_heads, key_dim, value_dim, g, b, q, k, v,
+                                ssm_state, out_values);
+    free(g); free(b);
+    return rc;
+}
+
+/* One whole Gated-DeltaNet layer step between the projections and o_proj, in
+ * the order of crates/moeflux-sys/metal_infer/infer.m:2625-2760 and of the GPU
+ * chain at crates/moeflux/src/riir/linear_attn_forward.rs:607-664:
+ * conv1d+SiLU over [q|k|v] channels, roll the conv state, per-head q/k norm,
+ * recurrence, gated RMS norm (weight shared by all v-heads).
+ *   qkv_in [C], C = 2*k_heads*key_dim + v_heads*value_dim; z [v_heads*value_dim];
+ *   conv_state [(K-1), C] and ssm_state [v_heads, value_dim, key_dim] mutated. */
+ORC_API int orc_gdn_step(int32_t k_heads, int32_t v_heads, int32_t key_dim,
+                         int32_t value_dim, int32_t kernel_size, float eps,
+                         const uint16_t *conv_w_bf16, const float *a_log,
+                         const uint16_t *dt_bias_bf16, const uint16_t *norm_w_bf16,
+                         const float *qkv_in, const float *z, const float *alpha,
+                         const float *beta, float *conv_state, float *ssm_state,
+                         float *out) {
+    if (!conv_w_bf16 || !a_log || !dt_bias_bf16 || !norm_w_bf16 || !qkv_in || !z ||
+        !alpha || !beta || !conv_state || !ssm_state || !out)
+        return -1;
+    if (k_heads <= 0 || v_heads <= 0 || key_dim <= 0 || value_dim <= 0 || kernel_size < 2)
+        return -1;
+    if (v_heads % k_heads != 0) return -1;
+    const int total_key = k_heads * key_dim;
+    const int total_value = v_heads * value_dim;
+    const int C = 2 * total_key + total_value;
+    float *conv_out = (float *)malloc((size_t)C * sizeof(float));
+    float *vals = (float *)malloc((size_t)total_value * sizeof(float));
+    if (!conv_out || !vals) { free(conv_out); free(vals); return -1; }
+    int rc = orc_conv1d_step(conv_state, qkv_in, conv_w_bf16, C, kernel_size, conv_out);
+    if (rc == 0) rc = orc_conv_state_shift(conv_state, qkv_in, C, kernel_size);
+    float *lin_q = conv_out, *lin_k = conv_out + total_key, *lin_v = conv_out + 2 * total_key;
+    if (rc == 0) rc = orc_rms_norm_qk(k_heads, key_dim, lin_q, lin_k);
+    if (rc == 0)
+        rc = orc_gated_delta_recurrence(a_log, dt_bias_bf16, alpha, beta, lin_q, lin_k, lin_v,
+                                        v_heads, k_heads, key_dim, value_dim, ssm_state, vals);
+    for (int vh = 0; rc == 0 && vh < v_heads; vh++)
+        rc = orc_rms_norm_gated(value_dim, eps, vals + (int64_t)vh * value_dim,
+                                z + (int64_t)vh * value_dim, norm_w_bf16,
+                                out + (int64_t)vh * value_dim);
+    free(conv_out); free(vals);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Prompt chunks: the reference has no batched prefill; eval_prompt is a      */
+/* token loop (crates/moeflux/src/riir/mod.rs:1196-1214), so a chunk is        */
+/* defined as that loop.                                                       */
+/* ------------------------------------------------------------------------ */
+
+/* Causal attention over a chunk of T new tokens appended after `kv_len0`
+ * cached positions: token t runs orc_sdpa with kv_len = kv_len0 + t + 1 (the
+ * current token attends to itself, full_attn_forward.rs:293,331).
+ *   q, q_gate, out: [T, Hq*d];  k_cache, v_cache: [kv_len0 + T, Hkv*d] already
+ *   holding the chunk's rows at positions kv_len0.. . */
+ORC_API int orc_prefill_attn(int32_t T, int32_t kv_len0, int32_t num_attn_heads,
+                             int32_t num_kv_heads, int32_t head_dim, const float *q,
+                             const float *q_gate, const float *k_cache,
+                             const float *v_cache, float *out) {
+    if (T <= 0 || kv_len0 < 0) return -1;
+    const int64_t q_dim = (int64_t)num_attn_heads * head_dim;
+    for (int t = 0; t < T; t++) {
+        int rc = orc_sdpa(kv_len0 + t + 1, num_attn_heads, num_kv_heads, head_dim,
+                          q + t * q_dim, q_gate + t * q_dim, k_cache, v_cache,
+                          out + t * q_dim);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+/* T sequential orc_gdn_step calls; inputs are [T, ...] row-major. */
+ORC_API int orc_prefill_gdn(int32_t T, int32_t k_heads, int32_t v_heads, int32_t key_dim,
+                            int32_t value_dim, int32_t kernel_size, float eps,
+                            const uint16_t *conv_w_bf16, const float *a_log,
+                            const uint16_t *dt_bias_bf16, const uint16_t *norm_w_bf16,
+                            const float *qkv_in, const float *z, const float *alpha,
+                            const float *beta, float *conv_state, float *ssm_state,
+                            float *out) {
+    if (T <= 0) return -1;
+    const int64_t C = 2 * (int64_t)k_heads * key_dim + (int64_t)v_heads * value_dim;
+    const int64_t tv = (int64_t)v_heads * value_dim;
+    for (int t = 0; t < T; t++) {
+        int rc = orc_gdn_step(k_heads, v_heads, key_dim, value_dim, kernel_size, eps,
+                              conv_w_bf16, a_log, dt_bias_bf16, norm_w_bf16,
+                              qkv_in + t * C, z + t * tv, alpha + (int64_t)t * v_heads,
+                              beta + (int64_t)t * v_heads, conv_state, ssm_state,
+                              out + t * tv);
+        if (rc) return rc;
+    }
+    return 0;
+}

@@ -1,0 +1,96 @@
+"""GPU parity of the Gated-DeltaNet path against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+from tests.util import TOL_F32, GdnCase, idx, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _ctx(mfa, case, num_layers=1):
+    from moeflux_amd import Config
+    c = mfa.Ctx(Config(num_layers=num_layers, full_attn_interval=num_layers + 1,
+                       linear_num_k_heads=case.Hk, linear_num_v_heads=case.Hv,
+                       linear_key_dim=case.dk, linear_value_dim=case.dv,
+                       conv_kernel_size=case.K, rms_norm_eps=case.eps))
+    for l in range(num_layers):
+        c.set_linear_weights(l, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+    return c
+
+
+@pytest.mark.parametrize("Hk,Hv,dk,dv", [(16, 32, 128, 128), (16, 64, 128, 128), (2, 2, 128, 128),
+                                          (4, 8, 64, 64), (1, 3, 128, 128)])
+def test_gdn_step_matches_oracle(mfa, Hk, Hv, dk, dv):
+    case = GdnCase(5 + Hv, Hk, Hv, dk, dv, T=6)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case) as c:
+        c.linear_state_import(0, case.conv_state, case.ssm_state)
+        for t in range(case.T):
+            out = c.gdn_step(0, case.qkv[t], case.z[t], case.alpha[t], case.beta[t])
+            assert rel_err(out, ref_out[t]) <= TOL_F32, f"step {t}"
+        conv, ssm = c.linear_state_export(0)
+    assert np.array_equal(conv.reshape(-1), ref_conv)  # the history is copied, never computed
+    assert rel_err(ssm, ref_ssm) <= TOL_F32
+
+
+def test_config2_from_zero_state_and_prefill(mfa):
+    """BASELINE config 2 shape with A_log = dt_bias = 0 and unit norm weight; the
+    chunk call equals the token loop."""
+    case = GdnCase(0xC0FFEE + 2, 16, 32, 128, 128, T=9, zero_state=True, plain=True)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case, num_layers=2) as c:
+        out = c.prefill_gdn(1, case.qkv, case.z, case.alpha, case.beta)
+        conv, ssm = c.linear_state_export(1)
+        conv0, ssm0 = c.linear_state_export(0)
+    assert rel_err(out, ref_out) <= TOL_F32
+    assert np.array_equal(conv.reshape(-1), ref_conv)
+    assert rel_err(ssm, ref_ssm) <= TOL_F32
+    assert not conv0.any() and not ssm0.any()  # the other layer is untouched
+
+
+def test_gdn_kernel_hooks(mfa, oracle):
+    """The five reference kernels one at a time (inputs of tests/diff_oracle.rs:2091-2260)."""
+    Hk, Hv, dk, dv, K = 16, 32, 128, 128, 4
+    case = GdnCase(3, Hk, Hv, dk, dv)
+    C = case.C
+    state = (np.sin(0.013 * idx(3 * C)) * 0.4 + 0.02).astype(np.float32)
+    x = (np.cos(0.019 * idx(C)) * 0.5 - 0.1).astype(np.float32)
+    out, rolled = mfa.conv1d_step(state, x, case.conv_w, C, K)
+    assert rel_err(out, oracle.conv1d_step(state, x, case.conv_w, C, K)) <= TOL_F32
+    assert np.array_equal(rolled, oracle.conv_state_shift(state, x, C, K))
+
+    q = (np.sin(0.011 * idx(Hk * dk)) * 0.4 + 0.05).astype(np.float32)
+    k = (np.cos(0.019 * idx(Hk * dk)) * 0.5 - 0.1).astype(np.float32)
+    v = (np.sin(0.023 * idx(Hv * dv)) * 0.6 + 0.02).astype(np.float32)
+    qn, kn = mfa.rms_norm_qk(Hk, dk, q, k)
+    qr, kr = oracle.rms_norm_qk(Hk, dk, q, k)
+    assert rel_err(qn, qr) <= TOL_F32 and rel_err(kn, kr) <= TOL_F32
+
+    xb = (np.sin(0.011 * idx(128)) * 0.6 + 0.05).astype(np.float32)
+    zb = (np.cos(0.017 * idx(128)) * 1.2 - 0.1).astype(np.float32)
+    assert rel_err(mfa.rms_norm_bare_cpu(xb, 1e-6), oracle.rms_norm_bare(xb, 1e-6)) <= TOL_F32
+    assert rel_err(mfa.rms_norm_gated_cpu(xb, zb, case.norm_w, 1e-6),
+                   oracle.rms_norm_gated(xb, zb, case.norm_w, 1e-6)) <= TOL_F32
+
+    alpha = (np.sin(0.013 * idx(Hv)) * 0.3).astype(np.float32)
+    beta = (np.cos(0.017 * idx(Hv)) * 0.5).astype(np.float32)
+    g, b = mfa.compute_decay_beta(alpha, beta, case.a_log, case.dt_bias)
+    gr, br = oracle.decay_beta(alpha, beta, case.a_log, case.dt_bias)
+    assert rel_err(g, gr) <= TOL_F32 and rel_err(b, br) <= TOL_F32
+
+    s1, o1 = mfa.gated_delta_net_step(Hv, Hk, dk, dv, gr, br, qr, kr, v, case.ssm_state)
+    s2, o2 = oracle.delta_net_step(Hv, Hk, dk, dv, gr, br, qr, kr, v, case.ssm_state)
+    assert rel_err(o1, o2) <= TOL_F32 and rel_err(s1, s2) <= TOL_F32
+
+    zero = np.zeros_like(case.ssm_state)  # the reference's test starts from a zero state
+    s1, o1 = mfa.gated_delta_recurrence_cpu(case.a_log, case.dt_bias, alpha, beta, qr, kr, v, Hv,
+                                            Hk, dk, dv, zero)
+    s2, o2 = oracle.gated_delta_recurrence(case.a_log, case.dt_bias, alpha, beta, qr, kr, v, Hv,
+                                           Hk, dk, dv, zero)
+    assert rel_err(o1, o2) <= TOL_F32 and rel_err(s1, s2) <= TOL_F32
+
+    z = case.z[0]
+    y1 = mfa.gated_rms_norm(Hv, dv, 1e-6, o2, z, case.norm_w)
+    y2 = np.concatenate([oracle.rms_norm_gated(o2[h * dv:(h + 1) * dv], z[h * dv:(h + 1) * dv],
+                                               case.norm_w, 1e-6) for h in range(Hv)])
+    assert rel_err(y1, y2) <= TOL_F32
