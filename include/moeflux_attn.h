@@ -98,6 +98,11 @@ int mfa_set_linear_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *conv_w_b
  * the reference checks tiled against single-shot MLA (tests/mla_sdpa_tiled.rs:
  * 176-216). */
 int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits);
+/* Measurement aid with no reference counterpart: when `on` is non-zero the
+ * decode entry points launch only the split-K partial kernel (no merge, `out`
+ * is not written), so that a timed loop isolates the kernel that streams the
+ * cache.  Default off. */
+int mfa_set_partial_only(mfa_ctx *ctx, int32_t on);
 
 /* ---- full attention: production path -------------------------------------- */
 

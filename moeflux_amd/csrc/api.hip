@@ -223,7 +223,7 @@ static int sdpa_decode_dev(Ctx *c, FullLayer *f, const float *q, const float *ga
     if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
     return launch_sdpa_decode(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
                               c->cfg.head_dim, f->len, c->plane_elems, f->k, f->v, q, gate, out,
-                              workspace(c), c->num_cus, c->forced_splits);
+                              workspace(c), c->num_cus, c->forced_splits, c->partial_only);
 }
 
 static int kv_append_dev(Ctx *c, FullLayer *f, const float *k, const float *v, int64_t rows) {
@@ -369,6 +369,13 @@ int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits) {
     if (!c) return fail(MFA_ERR_INVALID, "NULL context");
     if (num_splits < 0) return fail(MFA_ERR_INVALID, "num_splits must be >= 0");
     c->forced_splits = num_splits;
+    return MFA_OK;
+}
+
+int mfa_set_partial_only(mfa_ctx *ctx, int32_t on) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    c->partial_only = on ? 1 : 0;
     return MFA_OK;
 }
 

@@ -133,6 +133,7 @@ struct Ctx {
     float *part_ml = nullptr;
     size_t part_o_elems = 0, part_ml_elems = 0;
     int32_t forced_splits = 0;
+    int32_t partial_only = 0;
     // host-pointer staging
     float *stage = nullptr;
     size_t stage_elems = 0;
@@ -172,7 +173,7 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits);
 int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
                        size_t plane_elems, const void *k_tiled, const void *v_tiled,
                        const float *q, const float *gate, float *out, const SdpaWorkspace &ws,
-                       int num_cus, int forced_splits);
+                       int num_cus, int forced_splits, int partial_only = 0);
 // Scatter `n_rows` row-major rows ([n_rows, Hkv*D], f32 or bf16 source) into the
 // tiled planes starting at position pos0.
 int launch_kv_scatter(hipStream_t stream, int kv_dtype, int src_is_bf16, int Hkv, int D,

@@ -18,8 +18,13 @@
 //     bf16 caches use v_mfma_f32_16x16x32_bf16 with the f32 query and the f32
 //     probabilities each split into a bf16 high and low part (two
 //     instructions), which keeps the products exact to ~2^-17; f32 caches use
-//     v_mfma_f32_16x16x4_f32.  The four waves are merged through LDS and one
-//     (max, sum, O[16, D]) partial per workgroup is written.
+//     v_mfma_f32_16x16x4_f32.  The query (pre-multiplied by scale*log2 e, so
+//     that probabilities are single v_exp_f32) is converted once per
+//     workgroup into LDS in operand order.  The block's loads are issued in
+//     groups of eight into a ring of register buffers that is refilled for the
+//     next block as soon as a group has been consumed.  The four waves are
+//     merged through LDS and one (max, sum, O[16, D]) partial per workgroup is
+//     written.
 //   sdpa_merge_kernel    log-sum-exp merge of the partials, normalisation and
 //     the sigmoid gate.
 #include "mfa_internal.h"
@@ -27,125 +32,154 @@
 namespace mfa {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 static constexpr int kWaves = 4;
 static constexpr int kMaxSplits = 1024;
+static constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ inline float neg_inf() { return -__builtin_huge_valf(); }
-
 __device__ inline float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// x -> (hi, lo) with hi = bf16(x), lo = bf16(x - hi); x - hi is exact in f32.
-__device__ inline void split_bf16(float x, uint16_t &hi, uint16_t &lo) {
-    hi = f32_to_bf16_bits(x);
-    lo = f32_to_bf16_bits(x - bf16_bits_to_f32(hi));
+// (a, b) -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ inline uint32_t pack_bf16(float a, float b) {
+    f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
-
-union Pack8 {
-    uint16_t h[8];
-    uint4 u;
-    bf16x8 v;
-};
+// x = hi + lo + O(2^-17 x): hi = bf16(x), lo = bf16(x - hi); x - hi is exact in f32.
+__device__ inline void split_pair(float a, float b, uint32_t &hi, uint32_t &lo) {
+    hi = pack_bf16(a, b);
+    const float ah = __builtin_bit_cast(float, hi << 16);
+    const float bh = __builtin_bit_cast(float, hi & 0xffff0000u);
+    lo = pack_bf16(a - ah, b - bh);
+}
+__device__ inline bf16x8 as_bf16x8(uint4 u) { return __builtin_bit_cast(bf16x8, u); }
 
 template <typename KV, int D> struct Wave;
 
 // ---------------------------------------------------------------------------
-// bf16 cache
+// bf16 cache: blocks of 32 positions (64*D bytes of K and of V each)
 // ---------------------------------------------------------------------------
 template <int D> struct Wave<uint16_t, D> {
     static constexpr int BLK = 32;
-    static constexpr int KSTEPS = D / 32;  // MFMA steps per 16-position sub-tile
-    static constexpr int NACC = D / 16;
+    static constexpr int KSTEPS = D / 32;          // MFMA k-steps per 16-position sub-tile
+    static constexpr int NACC = D / 16;            // 16-wide output tiles of O^T
+    static constexpr int NLOAD = D / 16;           // 1 KiB loads per block, for K and for V alike
+    static constexpr int G = NLOAD < 8 ? NLOAD : 8;  // loads per register group
+    static constexpr int NG = NLOAD / G;           // groups per block for K, same for V
+    static constexpr int QLDS_U4 = KSTEPS * 2 * 64;
 
-    bf16x8 qhi[KSTEPS], qlo[KSTEPS];
-
-    __device__ void load_q(const float *qrow, bool ok, int g) {
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            Pack8 hi, lo;
-            float x[8];
-            if (ok) {
-                const float4 a = *(const float4 *)(qrow + 8 * (4 * s + g));
-                const float4 b = *(const float4 *)(qrow + 8 * (4 * s + g) + 4);
-                x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
-                x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; e++) x[e] = 0.f;
+    // Query operands in LDS: [k-step][hi|lo][lane] of 16 bytes.
+    __device__ static void prep_q(uint4 *qlds, const float *q, int kvh, int hg, int hpk, float qscale) {
+        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += kWaves * 64) {
+            const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
+            const int hin = hg * 16 + n;
+            uint4 hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+            if (hin < hpk) {
+                const float *p = q + (size_t)(kvh * hpk + hin) * D + 8 * (4 * s + g);
+                const float4 a = *(const float4 *)p, b = *(const float4 *)(p + 4);
+                split_pair(a.x * qscale, a.y * qscale, hi.x, lo.x);
+                split_pair(a.z * qscale, a.w * qscale, hi.y, lo.y);
+                split_pair(b.x * qscale, b.y * qscale, hi.z, lo.z);
+                split_pair(b.z * qscale, b.w * qscale, hi.w, lo.w);
             }
-#pragma unroll
-            for (int e = 0; e < 8; e++) split_bf16(x[e], hi.h[e], lo.h[e]);
-            qhi[s] = hi.v;
-            qlo[s] = lo.v;
+            qlds[(s * 2 + 0) * 64 + lane] = hi;
+            qlds[(s * 2 + 1) * 64 + lane] = lo;
         }
     }
 
-    struct Tile {
-        uint4 k[2][KSTEPS];
-        uint4 v[NACC];
+    struct Regs {
+        uint4 k[NG][G];
+        uint4 v[NG][G];
+    };
+    struct Scores {
+        f32x4 s[2];
     };
 
-    __device__ static void load_tile(Tile &t, const uint16_t *kplane, const uint16_t *vplane,
-                                     int64_t blk, int lane) {
-        const uint4 *kb = (const uint4 *)(kplane + blk * (int64_t)(BLK * D)) + lane;
-        const uint4 *vb = (const uint4 *)(vplane + blk * (int64_t)(BLK * D)) + lane;
+    __device__ static void load_k(Regs &r, int grp, const uint16_t *plane, int64_t blk, int lane) {
+        const uint4 *b = (const uint4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-        for (int sub = 0; sub < 2; sub++)
+        for (int i = 0; i < G; i++) r.k[grp][i] = b[i * 64];
+    }
+    __device__ static void load_v(Regs &r, int grp, const uint16_t *plane, int64_t blk, int lane) {
+        const uint4 *b = (const uint4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-            for (int s = 0; s < KSTEPS; s++) t.k[sub][s] = kb[(sub * KSTEPS + s) * 64];
-#pragma unroll
-        for (int dt = 0; dt < NACC; dt++) t.v[dt] = vb[dt * 64];
+        for (int i = 0; i < G; i++) r.v[grp][i] = b[i * 64];
     }
 
-    // One block of 32 positions.  lane = 16*g + n, n = head within the group.
-    __device__ void step(const Tile &t, int64_t blk, int64_t kv_len, float scale, int g,
-                         float &m_run, float &l_run, f32x4 (&o)[NACC]) {
-        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    __device__ static void zero_scores(Scores &sc) {
+        sc.s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        sc.s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // load index li = sub*KSTEPS + s
+    __device__ static void consume_k(const Regs &r, int grp, const uint4 *qlds, int lane, Scores &sc) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            Pack8 a0, a1;
-            a0.u = t.k[0][s];
-            a1.u = t.k[1][s];
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, qhi[s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, qhi[s], s1, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, qlo[s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, qlo[s], s1, 0, 0, 0);
+        for (int i = 0; i < G; i++) {
+            const int li = grp * G + i, sub = li / KSTEPS, s = li % KSTEPS;
+            const bf16x8 a = as_bf16x8(r.k[grp][i]);
+            const bf16x8 qh = as_bf16x8(qlds[(s * 2 + 0) * 64 + lane]);
+            const bf16x8 ql = as_bf16x8(qlds[(s * 2 + 1) * 64 + lane]);
+            sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qh, sc.s[sub], 0, 0, 0);
+            sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ql, sc.s[sub], 0, 0, 0);
         }
-        // Row 4g+i of sub-tile `sub` is position blk*32 + 16*sub + 4g + i.
-        float sc[8];
-        const int64_t base = blk * BLK + 4 * g;
+    }
+
+    struct Probs {
+        uint4 hi, lo;
+    };
+
+    // Row 4g+i of sub-tile `sub` is position blk*32 + 16*sub + 4g + i; scores are in
+    // log2 units.  Returns the rescale factor of the running state (1 if unchanged).
+    __device__ static float softmax(Scores &sc, int64_t blk, int64_t kv_len, int g, float &m_run,
+                                    float &l_run, Probs &p) {
+        float x[8];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            sc[i] = (base + i < kv_len) ? s0[i] * scale : neg_inf();
-            sc[4 + i] = (base + 16 + i < kv_len) ? s1[i] * scale : neg_inf();
+            x[i] = sc.s[0][i];
+            x[4 + i] = sc.s[1][i];
         }
-        float tmax = sc[0];
+        if ((blk + 1) * BLK > kv_len) {  // only the last block of the cache is ragged
+            const int64_t base = blk * BLK + 4 * g;
 #pragma unroll
-        for (int e = 1; e < 8; e++) tmax = fmaxf(tmax, sc[e]);
+            for (int i = 0; i < 4; i++) {
+                if (base + i >= kv_len) x[i] = neg_inf();
+                if (base + 16 + i >= kv_len) x[4 + i] = neg_inf();
+            }
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                           fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
         tmax = fmaxf(tmax, lane_xor(tmax, 16));
         tmax = fmaxf(tmax, lane_xor(tmax, 32));
         const float m_new = fmaxf(m_run, tmax);  // finite: position blk*32 is always valid
-        const float alpha = expf(m_run - m_new);
-        Pack8 phi, plo;
+        const float alpha = fast_exp2(m_run - m_new);
+        float e[8];
         float psum = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float p = expf(sc[e] - m_new);
-            psum += p;
-            split_bf16(p, phi.h[e], plo.h[e]);
+        for (int i = 0; i < 8; i++) {
+            e[i] = fast_exp2(x[i] - m_new);
+            psum += e[i];
         }
+        split_pair(e[0], e[1], p.hi.x, p.lo.x);
+        split_pair(e[2], e[3], p.hi.y, p.lo.y);
+        split_pair(e[4], e[5], p.hi.z, p.lo.z);
+        split_pair(e[6], e[7], p.hi.w, p.lo.w);
         l_run = l_run * alpha + psum;
         m_run = m_new;
+        return alpha;
+    }
+
+    __device__ static void consume_v(const Regs &r, int grp, const Probs &p, f32x4 (&o)[NACC]) {
+        const bf16x8 ph = as_bf16x8(p.hi), pl = as_bf16x8(p.lo);
 #pragma unroll
-        for (int dt = 0; dt < NACC; dt++) {
-            Pack8 a;
-            a.u = t.v[dt];
-            f32x4 acc = o[dt];
-            acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, phi.v, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, plo.v, acc, 0, 0, 0);
-            o[dt] = acc;
+        for (int i = 0; i < G; i++) {
+            const int dt = grp * G + i;
+            const bf16x8 a = as_bf16x8(r.v[grp][i]);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ph, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pl, o[dt], 0, 0, 0);
         }
     }
 
@@ -160,83 +194,107 @@ template <int D> struct Wave<uint16_t, D> {
 };
 
 // ---------------------------------------------------------------------------
-// f32 cache
+// f32 cache: blocks of 16 positions
 // ---------------------------------------------------------------------------
 template <int D> struct Wave<float, D> {
     static constexpr int BLK = 16;
-    static constexpr int KSTEPS = D / 16;  // 16-byte chunks per lane per block
+    static constexpr int KSTEPS = D / 16;  // 1 KiB loads of K per block (4 MFMAs each)
     static constexpr int NC = D / 64;
     static constexpr int NACC = D / 16;    // = NC * 4
+    static constexpr int NLOAD = D / 16;   // loads per block, for K and for V alike
+    static constexpr int G = NLOAD < 8 ? NLOAD : 8;
+    static constexpr int NG = NLOAD / G;
+    static constexpr int QLDS_U4 = KSTEPS * 64;
 
-    float4 qv[KSTEPS];
-
-    __device__ void load_q(const float *qrow, bool ok, int g) {
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            float4 z = {0.f, 0.f, 0.f, 0.f};
-            qv[s] = ok ? *(const float4 *)(qrow + 4 * (4 * s + g)) : z;
+    // Query operands in LDS: [k-step][lane] float4; lane (n, g) holds q[n][4(4s+g) .. +3].
+    __device__ static void prep_q(uint4 *qlds, const float *q, int kvh, int hg, int hpk, float qscale) {
+        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += kWaves * 64) {
+            const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
+            const int hin = hg * 16 + n;
+            float4 v = {0.f, 0.f, 0.f, 0.f};
+            if (hin < hpk) {
+                v = *(const float4 *)(q + (size_t)(kvh * hpk + hin) * D + 4 * (4 * s + g));
+                v.x *= qscale; v.y *= qscale; v.z *= qscale; v.w *= qscale;
+            }
+            qlds[slot] = __builtin_bit_cast(uint4, v);
         }
     }
 
-    struct Tile {
-        float4 k[KSTEPS];
-        float4 v[4][NC];
+    struct Regs {
+        float4 k[NG][G];
+        float4 v[NG][G];
+    };
+    struct Scores {
+        f32x4 s;
     };
 
-    __device__ static void load_tile(Tile &t, const float *kplane, const float *vplane,
-                                     int64_t blk, int lane) {
-        const float4 *kb = (const float4 *)(kplane + blk * (int64_t)(BLK * D)) + lane;
-        const float4 *vb = (const float4 *)(vplane + blk * (int64_t)(BLK * D)) + lane;
+    __device__ static void load_k(Regs &r, int grp, const float *plane, int64_t blk, int lane) {
+        const float4 *b = (const float4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-        for (int s = 0; s < KSTEPS; s++) t.k[s] = kb[s * 64];
+        for (int i = 0; i < G; i++) r.k[grp][i] = b[i * 64];
+    }
+    __device__ static void load_v(Regs &r, int grp, const float *plane, int64_t blk, int lane) {
+        const float4 *b = (const float4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int c = 0; c < NC; c++) t.v[i][c] = vb[(i * NC + c) * 64];
+        for (int i = 0; i < G; i++) r.v[grp][i] = b[i * 64];
     }
 
-    __device__ void step(const Tile &t, int64_t blk, int64_t kv_len, float scale, int g,
-                         float &m_run, float &l_run, f32x4 (&o)[NACC]) {
-        f32x4 s0 = {0.f, 0.f, 0.f, 0.f};
+    __device__ static void zero_scores(Scores &sc) { sc.s = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    __device__ static void consume_k(const Regs &r, int grp, const uint4 *qlds, int lane, Scores &sc) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[s].x, qv[s].x, s0, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[s].y, qv[s].y, s0, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[s].z, qv[s].z, s0, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(t.k[s].w, qv[s].w, s0, 0, 0, 0);
+        for (int i = 0; i < G; i++) {
+            const int s = grp * G + i;
+            const float4 a = r.k[grp][i];
+            const float4 b = __builtin_bit_cast(float4, qlds[s * 64 + lane]);
+            sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, sc.s, 0, 0, 0);
+            sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, sc.s, 0, 0, 0);
+            sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, sc.s, 0, 0, 0);
+            sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, sc.s, 0, 0, 0);
         }
-        float sc[4];
-        const int64_t base = blk * BLK + 4 * g;
+    }
+
+    struct Probs {
+        float p[4];
+    };
+
+    __device__ static float softmax(Scores &sc, int64_t blk, int64_t kv_len, int g, float &m_run,
+                                    float &l_run, Probs &p) {
+        float x[4] = {sc.s[0], sc.s[1], sc.s[2], sc.s[3]};
+        if ((blk + 1) * BLK > kv_len) {
+            const int64_t base = blk * BLK + 4 * g;
 #pragma unroll
-        for (int i = 0; i < 4; i++) sc[i] = (base + i < kv_len) ? s0[i] * scale : neg_inf();
-        float tmax = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            for (int i = 0; i < 4; i++)
+                if (base + i >= kv_len) x[i] = neg_inf();
+        }
+        float tmax = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
         tmax = fmaxf(tmax, lane_xor(tmax, 16));
         tmax = fmaxf(tmax, lane_xor(tmax, 32));
         const float m_new = fmaxf(m_run, tmax);
-        const float alpha = expf(m_run - m_new);
-        float p[4];
+        const float alpha = fast_exp2(m_run - m_new);
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            p[i] = expf(sc[i] - m_new);
-            psum += p[i];
+            p.p[i] = fast_exp2(x[i] - m_new);
+            psum += p.p[i];
         }
         l_run = l_run * alpha + psum;
         m_run = m_new;
+        return alpha;
+    }
+
+    // load index li = i*NC + c: MFMA set i contracts positions 4g+i; accumulator 4c+j
+    // collects d = 64c + 4m + j.
+    __device__ static void consume_v(const Regs &r, int grp, const Probs &p, f32x4 (&o)[NACC]) {
 #pragma unroll
-        for (int a = 0; a < NACC; a++) {
-            o[a][0] *= alpha; o[a][1] *= alpha; o[a][2] *= alpha; o[a][3] *= alpha;
+        for (int x = 0; x < G; x++) {
+            const int li = grp * G + x, i = li / NC, c = li % NC;
+            const float4 a = r.v[grp][x];
+            o[4 * c + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, p.p[i], o[4 * c + 0], 0, 0, 0);
+            o[4 * c + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, p.p[i], o[4 * c + 1], 0, 0, 0);
+            o[4 * c + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, p.p[i], o[4 * c + 2], 0, 0, 0);
+            o[4 * c + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, p.p[i], o[4 * c + 3], 0, 0, 0);
         }
-        // accumulator 4c+j collects d = 64c + 4m + j; MFMA set i contracts positions 4g+i.
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int c = 0; c < NC; c++) {
-                o[4 * c + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.v[i][c].x, p[i], o[4 * c + 0], 0, 0, 0);
-                o[4 * c + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.v[i][c].y, p[i], o[4 * c + 1], 0, 0, 0);
-                o[4 * c + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.v[i][c].z, p[i], o[4 * c + 2], 0, 0, 0);
-                o[4 * c + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(t.v[i][c].w, p[i], o[4 * c + 3], 0, 0, 0);
-            }
     }
 
     // accumulator 4c+j, lane group g, element i holds d = 64c + 16g + 4i + j
@@ -252,23 +310,24 @@ template <int D> struct Wave<float, D> {
 };
 
 // part_o:  [kv head][head group][split][16 heads][D]
-// part_ml: [kv head][head group][split][2][16]   (max, then sum)
+// part_ml: [kv head][head group][split][2][16]   (max in log2 units, then sum)
 template <typename KV, int D>
 __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
-    const float *__restrict__ q, int hpk, int64_t kv_len, int blocks_per_split, float scale,
+    const float *__restrict__ q, int hpk, int64_t kv_len, int blocks_per_split, float qscale,
     float *__restrict__ part_o, float *__restrict__ part_ml) {
     using W = Wave<KV, D>;
     constexpr int NACC = W::NACC;
+    constexpr int NG = W::NG;
+    __shared__ uint4 qlds[W::QLDS_U4];
+    __shared__ float sm[kWaves][16];
+    __shared__ float sl[kWaves][16];
+    __shared__ f32x4 red[2][NACC][64];
+
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, hg = blockIdx.y, kvh = blockIdx.z;
     const int nsplit = gridDim.x, nhg = gridDim.y;
-
-    const int head_in_kv = hg * 16 + n;
-    const bool head_ok = head_in_kv < hpk;
-    W w;
-    w.load_q(q + (int64_t)(kvh * hpk + (head_ok ? head_in_kv : 0)) * D, head_ok, g);
 
     const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
     const KV *vplane = v_tiled + (size_t)kvh * plane_elems;
@@ -277,38 +336,58 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     int64_t b1 = b0 + blocks_per_split;
     if (b1 > nblk) b1 = nblk;
 
+    // The first block's loads go out before anything else; the query conversion
+    // below overlaps their latency.
+    typename W::Regs r;
+    int64_t b = b0 + wave;
+    if (b < b1) {
+#pragma unroll
+        for (int x = 0; x < NG; x++) W::load_k(r, x, kplane, b, lane);
+#pragma unroll
+        for (int x = 0; x < NG; x++) W::load_v(r, x, vplane, b, lane);
+    }
+    W::prep_q(qlds, q, kvh, hg, hpk, qscale);
+    __syncthreads();
+
     f32x4 o[NACC];
 #pragma unroll
     for (int a = 0; a < NACC; a++) o[a] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = neg_inf(), l_run = 0.f;
 
-    // Two tiles in flight: the loads of block b+4 are issued before block b is consumed.
-    typename W::Tile t0, t1;
-    int64_t b = b0 + wave;
-    if (b < b1) W::load_tile(t0, kplane, vplane, b, lane);
-    while (b < b1) {
+    for (; b < b1; b += kWaves) {
         const int64_t bn = b + kWaves;
-        if (bn < b1) W::load_tile(t1, kplane, vplane, bn, lane);
-        w.step(t0, b, kv_len, scale, g, m_run, l_run, o);
-        if (bn >= b1) break;
-        const int64_t bnn = bn + kWaves;
-        if (bnn < b1) W::load_tile(t0, kplane, vplane, bnn, lane);
-        w.step(t1, bn, kv_len, scale, g, m_run, l_run, o);
-        b = bnn;
+        const bool more = bn < b1;
+        typename W::Scores sc;
+        W::zero_scores(sc);
+#pragma unroll
+        for (int x = 0; x < NG; x++) {
+            W::consume_k(r, x, qlds, lane, sc);
+            if (more) W::load_k(r, x, kplane, bn, lane);
+        }
+        typename W::Probs p;
+        const float alpha = W::softmax(sc, b, kv_len, g, m_run, l_run, p);
+        if (__any(alpha != 1.0f)) {  // the running max moved: rescale what has been accumulated
+#pragma unroll
+            for (int a = 0; a < NACC; a++) {
+                o[a][0] *= alpha; o[a][1] *= alpha; o[a][2] *= alpha; o[a][3] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < NG; x++) {
+            W::consume_v(r, x, p, o);
+            if (more) W::load_v(r, x, vplane, bn, lane);
+        }
     }
     l_run += lane_xor(l_run, 16);
     l_run += lane_xor(l_run, 32);
 
     // ---- merge the four waves ------------------------------------------------
-    __shared__ float sm[kWaves][16];
-    __shared__ float sl[kWaves][16];
-    __shared__ f32x4 red[2][NACC][64];
     if (g == 0) sm[wave][n] = m_run;
     __syncthreads();
     float M = sm[0][n];
 #pragma unroll
     for (int x = 1; x < kWaves; x++) M = fmaxf(M, sm[x][n]);
-    const float f = (m_run == neg_inf()) ? 0.f : expf(m_run - M);
+    const float f = (m_run == neg_inf()) ? 0.f : fast_exp2(m_run - M);
     l_run *= f;
 #pragma unroll
     for (int a = 0; a < NACC; a++) {
@@ -323,8 +402,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     if (wave < 2) {
 #pragma unroll
         for (int a = 0; a < NACC; a++) {
-            const f32x4 r = red[wave][a][lane];
-            o[a][0] += r[0]; o[a][1] += r[1]; o[a][2] += r[2]; o[a][3] += r[3];
+            const f32x4 t = red[wave][a][lane];
+            o[a][0] += t[0]; o[a][1] += t[1]; o[a][2] += t[2]; o[a][3] += t[3];
         }
     }
     __syncthreads();
@@ -336,8 +415,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     if (wave == 0) {
 #pragma unroll
         for (int a = 0; a < NACC; a++) {
-            const f32x4 r = red[0][a][lane];
-            o[a][0] += r[0]; o[a][1] += r[1]; o[a][2] += r[2]; o[a][3] += r[3];
+            const f32x4 t = red[0][a][lane];
+            o[a][0] += t[0]; o[a][1] += t[1]; o[a][2] += t[2]; o[a][3] += t[3];
         }
         const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
         W::store_o(part_o + (pid * 16 + n) * D, g, o);
@@ -348,54 +427,57 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     }
 }
 
-// grid (Hq, D/32), 256 threads: 32 output elements x 8 split lanes.
+// grid (Hq, D/64), 256 threads: 16 lanes x float4 cover 64 outputs of one split's row,
+// 16 such rows per pass.
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
     __shared__ float wsh[kMaxSplits];
-    __shared__ float redf[256];
+    __shared__ float redf[4];
+    __shared__ float4 acc4[16][16];
     const int h = blockIdx.x;
     const int kvh = h / hpk, hin = h % hpk, hg = hin / 16, n = hin % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
+    const int dl = tid & 15, sg = tid >> 4;  // 16 float4 lanes x 16 split lanes
+    const int d0 = blockIdx.y * 64 + dl * 4;
     float m = neg_inf();
     for (int s = tid; s < nsplit; s += 256) m = fmaxf(m, part_ml[(pid0 + s) * 32 + n]);
-    redf[tid] = m;
+#pragma unroll
+    for (int x = 1; x < 64; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
+    if (lane == 0) redf[wave] = m;
     __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-        if (tid < w) redf[tid] = fmaxf(redf[tid], redf[tid + w]);
-        __syncthreads();
-    }
-    const float M = redf[0];
+    const float M = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
     __syncthreads();
     float den = 0.f;
     for (int s = tid; s < nsplit; s += 256) {
         const float ms = part_ml[(pid0 + s) * 32 + n];
-        const float ws = (ms == neg_inf()) ? 0.f : expf(ms - M);
+        const float ws = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
         wsh[s] = ws;
         den += ws * part_ml[(pid0 + s) * 32 + 16 + n];
     }
-    redf[tid] = den;
+#pragma unroll
+    for (int x = 1; x < 64; x <<= 1) den += __shfl_xor(den, x, 64);
+    if (lane == 0) redf[wave] = den;
     __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-        if (tid < w) redf[tid] += redf[tid + w];
-        __syncthreads();
-    }
-    den = redf[0];
-    __syncthreads();
+    den = redf[0] + redf[1] + redf[2] + redf[3];
 
-    const int dl = tid & 31, sl = tid >> 5;
-    const int d = blockIdx.y * 32 + dl;
-    float acc = 0.f;
-    for (int s = sl; s < nsplit; s += 8)
-        acc += wsh[s] * part_o[((pid0 + s) * 16 + n) * D + d];
-    redf[tid] = acc;
+    float4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = sg; s < nsplit; s += 16) {
+        const float w = wsh[s];
+        const float4 v = *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0);
+        acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+    }
+    acc4[sg][dl] = acc;
     __syncthreads();
-    if (sl == 0) {
+    if (tid < 64) {
+        // thread -> one scalar output: float4 lane tid/4, component tid%4
+        const int ql = tid >> 2, qc = tid & 3;
         float t = 0.f;
 #pragma unroll
-        for (int x = 0; x < 8; x++) t += redf[x * 32 + dl];
+        for (int x = 0; x < 16; x++) t += ((const float *)&acc4[x][ql])[qc];
+        const int d = blockIdx.y * 64 + tid;
         const float gt = 1.0f / (1.0f + expf(-gate[(size_t)h * D + d]));
         out[(size_t)h * D + d] = (t / den) * gt;
     }
@@ -473,7 +555,6 @@ bool sdpa_shape_supported(int kv_dtype, int head_dim) {
 
 static int blk_of(int kv_dtype) { return kv_dtype == MFA_KV_BF16 ? 32 : 16; }
 
-// Returns blocks-per-split through *bps.
 int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced) {
     (void)D;
     const int hpk = Hq / Hkv;
@@ -508,16 +589,16 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits) {
 template <typename KV, int D>
 static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
                            size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
-                           float scale, float *po, float *pml) {
+                           float qscale, float *po, float *pml) {
     hipLaunchKernelGGL((sdpa_partial_kernel<KV, D>), grid, dim3(kWaves * 64), 0, stream,
-                       (const KV *)k, (const KV *)v, plane_elems, q, hpk, kv_len, bps, scale, po,
+                       (const KV *)k, (const KV *)v, plane_elems, q, hpk, kv_len, bps, qscale, po,
                        pml);
 }
 
 int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
                        size_t plane_elems, const void *k_tiled, const void *v_tiled,
                        const float *q, const float *gate, float *out, const SdpaWorkspace &ws,
-                       int num_cus, int forced_splits) {
+                       int num_cus, int forced_splits, int partial_only) {
     if (!sdpa_shape_supported(kv_dtype, D))
         return fail(MFA_ERR_SHAPE, "sdpa: head_dim %d / kv dtype %d not supported", D, kv_dtype);
     if (kv_len <= 0) return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld)", (long long)kv_len);
@@ -533,11 +614,12 @@ int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D,
     const int64_t bps = bps_for(kv_dtype, kv_len, splits);
     const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
     splits = (int)((nblk + bps - 1) / bps);
-    const float scale = 1.0f / sqrtf((float)D);
+    // scores are produced in log2 units: q is pre-multiplied by (1/sqrt(D)) * log2(e)
+    const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     dim3 grid(splits, nhg, Hkv);
 #define MFA_LAUNCH(KV, DD)                                                                      \
     launch_partial<KV, DD>(stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, kv_len, (int)bps, \
-                           scale, ws.part_o, ws.part_ml)
+                           qscale, ws.part_o, ws.part_ml)
     if (kv_dtype == MFA_KV_BF16) {
         if (D == 64) MFA_LAUNCH(uint16_t, 64);
         else if (D == 128) MFA_LAUNCH(uint16_t, 128);
@@ -549,7 +631,8 @@ int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D,
     }
 #undef MFA_LAUNCH
     MFA_HIP(hipGetLastError());
-    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(Hq, D / 32), dim3(256), 0, stream, ws.part_o,
+    if (partial_only) return MFA_OK;
+    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(Hq, D / 64), dim3(256), 0, stream, ws.part_o,
                        ws.part_ml, splits, hpk, nhg, D, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
