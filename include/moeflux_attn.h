@@ -258,6 +258,20 @@ int mfa_gated_delta_recurrence(const float *a_log, const uint16_t *dt_bias_bf16,
 int mfa_gated_rms_norm(int32_t num_heads, int32_t dim, float eps, const float *x,
                        const float *z, const uint16_t *weight_bf16, float *out);
 
+/* ---- diagnostics (host only, no GPU needed) --------------------------------- */
+/* No counterpart in the reference.  The device KV cache is not row-major (it is
+ * stored in the order the decode kernel's matrix-instruction operands consume
+ * it); these two functions expose the host-side arithmetic so that it can be
+ * tested without a GPU.
+ * Element offset, inside one kv head's plane, of channel x of position pos
+ * (is_v selects the V plane's order); -1 on a bad argument. */
+int64_t mfa_debug_kv_offset(int32_t kv_dtype, int32_t is_v, int64_t pos, int32_t x,
+                            int32_t head_dim);
+/* Number of split-K partitions the decode launcher uses for this shape. */
+int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t num_attn_heads, int32_t num_kv_heads,
+                             int32_t head_dim, int64_t kv_len, int32_t num_cus,
+                             int32_t forced_splits);
+
 #pragma GCC visibility pop
 
 #ifdef __cplusplus

@@ -660,6 +660,23 @@ int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state
     return MFA_OK;
 }
 
+/* ---- diagnostics --------------------------------------------------------------------- */
+
+int64_t mfa_debug_kv_offset(int32_t kv_dtype, int32_t is_v, int64_t pos, int32_t x, int32_t D) {
+    if (!sdpa_shape_supported(kv_dtype, D) || pos < 0 || x < 0 || x >= D) return -1;
+    if (kv_dtype == MFA_KV_BF16)
+        return is_v ? KvTile<uint16_t>::v_off(pos, x, D) : KvTile<uint16_t>::k_off(pos, x, D);
+    return is_v ? KvTile<float>::v_off(pos, x, D) : KvTile<float>::k_off(pos, x, D);
+}
+
+int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t Hq, int32_t Hkv, int32_t D, int64_t kv_len,
+                             int32_t num_cus, int32_t forced_splits) {
+    if (!sdpa_shape_supported(kv_dtype, D) || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || kv_len <= 0 ||
+        num_cus <= 0)
+        return -1;
+    return sdpa_pick_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced_splits);
+}
+
 /* ---- timing ------------------------------------------------------------------------ */
 
 int mfa_timer_start(mfa_ctx *ctx) {

@@ -1,0 +1,75 @@
+"""Host-side arithmetic of the library that needs no GPU: the tiled KV-cache
+addressing and the split-K partitioning."""
+import numpy as np
+import pytest
+
+from moeflux_amd import ffi
+
+
+@pytest.mark.parametrize("dtype,blk", [(ffi.KV_BF16, 32), (ffi.KV_F32, 16)])
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("is_v", [0, 1])
+def test_tiling_is_a_bijection_on_every_block(dtype, blk, D, is_v):
+    lib = ffi.load()
+    npos = 3 * blk
+    off = np.array([[lib.mfa_debug_kv_offset(dtype, is_v, p, x, D) for x in range(D)]
+                    for p in range(npos)])
+    assert sorted(off.reshape(-1).tolist()) == list(range(npos * D))        # one-to-one, no holes
+    for b in range(3):                                                       # a block is contiguous
+        o = off[b * blk:(b + 1) * blk]
+        assert o.min() == b * blk * D and o.max() == (b + 1) * blk * D - 1
+
+
+def test_tiling_matches_the_decode_kernels_operand_order():
+    """bf16: lane (row m = lane%16, group g = lane/16) of load `li` in a block reads 8
+    consecutive elements at li*512 + lane*8; they must be channels 8*(4s+g)..+7 of position
+    16*sub + m for K (li = sub*D/32 + s), and for V the 8 positions
+    {4g..4g+3, 16+4g..16+4g+3} of channel 16*dt + m (li = dt)."""
+    lib = ffi.load()
+    D = 256
+    for li in (0, 5, 9, 15):
+        for lane in (0, 17, 38, 63):
+            m, g = lane % 16, lane // 16
+            base = li * 512 + lane * 8
+            sub, s = li // (D // 32), li % (D // 32)
+            for e in range(8):
+                assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, 16 * sub + m, 8 * (4 * s + g) + e, D) == base + e
+                pos = 16 * (e // 4) + 4 * g + e % 4
+                assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 1, pos, 16 * li + m, D) == base + e
+    # f32: K load s holds channels 4*(4s+g)..+3 of position m; V load li = i*NC + c holds
+    # channels 64c + 4m .. +3 of position 4g + i
+    D = 128
+    for li in (0, 3, 7):
+        for lane in (0, 21, 63):
+            m, g = lane % 16, lane // 16
+            base = li * 256 + lane * 4
+            i, c = li // (D // 64), li % (D // 64)
+            for j in range(4):
+                assert lib.mfa_debug_kv_offset(ffi.KV_F32, 0, m, 4 * (4 * li + g) + j, D) == base + j
+                assert lib.mfa_debug_kv_offset(ffi.KV_F32, 1, 4 * g + i, 64 * c + 4 * m + j, D) == base + j
+
+
+def test_tiling_rejects_bad_arguments():
+    lib = ffi.load()
+    assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, -1, 0, 256) == -1
+    assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, 0, 256, 256) == -1
+    assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, 0, 0, 100) == -1
+    assert lib.mfa_debug_kv_offset(9, 0, 0, 0, 256) == -1
+
+
+def test_split_partitioning():
+    lib = ffi.load()
+    ns = lib.mfa_debug_num_splits
+    # config 3: 1024 blocks of 32 positions per kv head, 256 CUs / 2 kv heads -> 128 splits
+    assert ns(ffi.KV_BF16, 32, 2, 256, 32768, 256, 0) == 128
+    # config 1: 256 blocks of 16 positions per kv head, 4 kv heads -> 64 splits of 4 blocks
+    assert ns(ffi.KV_F32, 32, 4, 128, 4096, 256, 0) == 64
+    assert ns(ffi.KV_BF16, 32, 2, 256, 1, 256, 0) == 1
+    assert ns(ffi.KV_BF16, 32, 2, 256, 33, 256, 0) == 1          # 2 blocks, one split
+    for forced in (1, 2, 7, 64):
+        got = ns(ffi.KV_BF16, 32, 2, 256, 8192, 256, forced)
+        assert 1 <= got <= forced
+    # more than 16 query heads per kv head: head groups share the CUs
+    assert ns(ffi.KV_BF16, 64, 2, 128, 32768, 256, 0) == 64
+    assert ns(ffi.KV_BF16, 30, 4, 128, 64, 256, 0) == -1          # 30 % 4 != 0
+    assert ns(ffi.KV_BF16, 32, 2, 256, 0, 256, 0) == -1
