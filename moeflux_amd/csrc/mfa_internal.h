@@ -56,7 +56,7 @@ __host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 // (32 positions for bf16, 16 for f32); a block of one plane is contiguous.
 //
 // bf16, block of 32 positions, element (p, x) with p in [0,32), x in [0,D):
-//   K: [sub = p/16][chunk = x/8][row = p%16][e = x%8]
+//   K: [step = x/32][sub = p/16][chunk = (x%32)/8][row = p%16][e = x%8]
 //   V: [dt = x/16][g = (p%16)/4][m = x%16][e = 4*(p/16) + p%4]
 // f32, block of 16 positions:
 //   K: [chunk = x/4][row = p][e = x%4]
@@ -68,7 +68,7 @@ template <> struct KvTile<uint16_t> {
     __host__ __device__ static inline int64_t k_off(int64_t pos, int x, int D) {
         const int64_t blk = pos / 32;
         const int p = (int)(pos % 32);
-        return blk * 32 * D + ((int64_t)(p / 16) * (D / 8) + x / 8) * 128 + (p % 16) * 8 + (x % 8);
+        return blk * 32 * D + (((int64_t)(x / 32) * 2 + p / 16) * 4 + (x % 32) / 8) * 128 + (p % 16) * 8 + (x % 8);
     }
     __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
         const int64_t blk = pos / 32;

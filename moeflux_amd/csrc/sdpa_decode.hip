@@ -6,7 +6,7 @@
 // crates/moeflux/src/riir/linear_attn_forward.rs:850-902) and its CPU fallback
 // sdpa_cpu (crates/moeflux/src/riir/sdpa.rs:63-172) with two launches:
 //
-//   sdpa_partial_kernel  grid (splits, head groups, kv heads), 4 waves each.
+//   sdpa_partial_kernel  grid (splits, head groups, kv heads), 4 or 8 waves each.
 //     A wave streams whole position blocks of its kv head's K and V planes
 //     exactly once, each wave-level load being a contiguous 1 KiB run that
 //     lands directly in MFMA operand registers (see KvTile in mfa_internal.h).
@@ -20,11 +20,11 @@
 //     instructions), which keeps the products exact to ~2^-17; f32 caches use
 //     v_mfma_f32_16x16x4_f32.  The query (pre-multiplied by scale*log2 e, so
 //     that probabilities are single v_exp_f32) is converted once per
-//     workgroup into LDS in operand order.  The block's loads are issued in
-//     groups of eight into a ring of register buffers that is refilled for the
-//     next block as soon as a group has been consumed.  The four waves are
-//     merged through LDS and one (max, sum, O[16, D]) partial per workgroup is
-//     written.
+//     workgroup into LDS in operand order.  A block's K and V are a stream of
+//     groups of up to eight 1 KiB loads; two register buffers alternate, the
+//     one just consumed being refilled with the group after next.  The waves
+//     are merged through LDS and one (max, sum, O[16, D]) partial per
+//     workgroup is written.
 //   sdpa_merge_kernel    log-sum-exp merge of the partials, normalisation and
 //     the sigmoid gate.
 #include "mfa_internal.h"
@@ -36,7 +36,6 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-static constexpr int kWaves = 4;
 static constexpr int kMaxSplits = 1024;
 static constexpr float kLog2e = 1.4426950408889634f;
 
@@ -74,7 +73,7 @@ template <int D> struct Wave<uint16_t, D> {
 
     // Query operands in LDS: [k-step][hi|lo][lane] of 16 bytes.
     __device__ static void prep_q(uint4 *qlds, const float *q, int kvh, int hg, int hpk, float qscale) {
-        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += kWaves * 64) {
+        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += blockDim.x) {
             const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
             const int hin = hg * 16 + n;
             uint4 hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
@@ -91,23 +90,18 @@ template <int D> struct Wave<uint16_t, D> {
         }
     }
 
-    struct Regs {
-        uint4 k[NG][G];
-        uint4 v[NG][G];
-    };
     struct Scores {
         f32x4 s[2];
     };
+    struct Probs {
+        uint4 hi, lo;
+    };
 
-    __device__ static void load_k(Regs &r, int grp, const uint16_t *plane, int64_t blk, int lane) {
+    // group `grp` of a block: loads grp*G .. grp*G+G-1 of the block's contiguous run
+    __device__ static void load_group(uint4 (&dst)[G], const uint16_t *plane, int64_t blk, int grp, int lane) {
         const uint4 *b = (const uint4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-        for (int i = 0; i < G; i++) r.k[grp][i] = b[i * 64];
-    }
-    __device__ static void load_v(Regs &r, int grp, const uint16_t *plane, int64_t blk, int lane) {
-        const uint4 *b = (const uint4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
-#pragma unroll
-        for (int i = 0; i < G; i++) r.v[grp][i] = b[i * 64];
+        for (int i = 0; i < G; i++) dst[i] = b[i * 64];
     }
 
     __device__ static void zero_scores(Scores &sc) {
@@ -115,22 +109,18 @@ template <int D> struct Wave<uint16_t, D> {
         sc.s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // load index li = sub*KSTEPS + s
-    __device__ static void consume_k(const Regs &r, int grp, const uint4 *qlds, int lane, Scores &sc) {
+    // load index li = 2*s + sub: both sub-tiles of a k-step share one read of the query operands
+    __device__ static void consume_k(const uint4 (&src)[G], int grp, const uint4 *qlds, int lane, Scores &sc) {
 #pragma unroll
         for (int i = 0; i < G; i++) {
-            const int li = grp * G + i, sub = li / KSTEPS, s = li % KSTEPS;
-            const bf16x8 a = as_bf16x8(r.k[grp][i]);
+            const int li = grp * G + i, s = li / 2, sub = li % 2;
+            const bf16x8 a = as_bf16x8(src[i]);
             const bf16x8 qh = as_bf16x8(qlds[(s * 2 + 0) * 64 + lane]);
             const bf16x8 ql = as_bf16x8(qlds[(s * 2 + 1) * 64 + lane]);
             sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qh, sc.s[sub], 0, 0, 0);
             sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ql, sc.s[sub], 0, 0, 0);
         }
     }
-
-    struct Probs {
-        uint4 hi, lo;
-    };
 
     // Row 4g+i of sub-tile `sub` is position blk*32 + 16*sub + 4g + i; scores are in
     // log2 units.  Returns the rescale factor of the running state (1 if unchanged).
@@ -172,12 +162,12 @@ template <int D> struct Wave<uint16_t, D> {
         return alpha;
     }
 
-    __device__ static void consume_v(const Regs &r, int grp, const Probs &p, f32x4 (&o)[NACC]) {
+    __device__ static void consume_v(const uint4 (&src)[G], int grp, const Probs &p, f32x4 (&o)[NACC]) {
         const bf16x8 ph = as_bf16x8(p.hi), pl = as_bf16x8(p.lo);
 #pragma unroll
         for (int i = 0; i < G; i++) {
             const int dt = grp * G + i;
-            const bf16x8 a = as_bf16x8(r.v[grp][i]);
+            const bf16x8 a = as_bf16x8(src[i]);
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, ph, o[dt], 0, 0, 0);
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pl, o[dt], 0, 0, 0);
         }
@@ -194,7 +184,7 @@ template <int D> struct Wave<uint16_t, D> {
 };
 
 // ---------------------------------------------------------------------------
-// f32 cache: blocks of 16 positions
+// f32 cache: blocks of 16 positions (64*D bytes of K and of V each)
 // ---------------------------------------------------------------------------
 template <int D> struct Wave<float, D> {
     static constexpr int BLK = 16;
@@ -208,7 +198,7 @@ template <int D> struct Wave<float, D> {
 
     // Query operands in LDS: [k-step][lane] float4; lane (n, g) holds q[n][4(4s+g) .. +3].
     __device__ static void prep_q(uint4 *qlds, const float *q, int kvh, int hg, int hpk, float qscale) {
-        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += kWaves * 64) {
+        for (int slot = threadIdx.x; slot < KSTEPS * 64; slot += blockDim.x) {
             const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
             const int hin = hg * 16 + n;
             float4 v = {0.f, 0.f, 0.f, 0.f};
@@ -220,32 +210,26 @@ template <int D> struct Wave<float, D> {
         }
     }
 
-    struct Regs {
-        float4 k[NG][G];
-        float4 v[NG][G];
-    };
     struct Scores {
         f32x4 s;
     };
+    struct Probs {
+        float p[4];
+    };
 
-    __device__ static void load_k(Regs &r, int grp, const float *plane, int64_t blk, int lane) {
-        const float4 *b = (const float4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
+    __device__ static void load_group(uint4 (&dst)[G], const float *plane, int64_t blk, int grp, int lane) {
+        const uint4 *b = (const uint4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
 #pragma unroll
-        for (int i = 0; i < G; i++) r.k[grp][i] = b[i * 64];
-    }
-    __device__ static void load_v(Regs &r, int grp, const float *plane, int64_t blk, int lane) {
-        const float4 *b = (const float4 *)(plane + blk * (int64_t)(BLK * D)) + lane + grp * G * 64;
-#pragma unroll
-        for (int i = 0; i < G; i++) r.v[grp][i] = b[i * 64];
+        for (int i = 0; i < G; i++) dst[i] = b[i * 64];
     }
 
     __device__ static void zero_scores(Scores &sc) { sc.s = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-    __device__ static void consume_k(const Regs &r, int grp, const uint4 *qlds, int lane, Scores &sc) {
+    __device__ static void consume_k(const uint4 (&src)[G], int grp, const uint4 *qlds, int lane, Scores &sc) {
 #pragma unroll
         for (int i = 0; i < G; i++) {
             const int s = grp * G + i;
-            const float4 a = r.k[grp][i];
+            const float4 a = __builtin_bit_cast(float4, src[i]);
             const float4 b = __builtin_bit_cast(float4, qlds[s * 64 + lane]);
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, sc.s, 0, 0, 0);
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, sc.s, 0, 0, 0);
@@ -253,10 +237,6 @@ template <int D> struct Wave<float, D> {
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, sc.s, 0, 0, 0);
         }
     }
-
-    struct Probs {
-        float p[4];
-    };
 
     __device__ static float softmax(Scores &sc, int64_t blk, int64_t kv_len, int g, float &m_run,
                                     float &l_run, Probs &p) {
@@ -285,11 +265,11 @@ template <int D> struct Wave<float, D> {
 
     // load index li = i*NC + c: MFMA set i contracts positions 4g+i; accumulator 4c+j
     // collects d = 64c + 4m + j.
-    __device__ static void consume_v(const Regs &r, int grp, const Probs &p, f32x4 (&o)[NACC]) {
+    __device__ static void consume_v(const uint4 (&src)[G], int grp, const Probs &p, f32x4 (&o)[NACC]) {
 #pragma unroll
         for (int x = 0; x < G; x++) {
             const int li = grp * G + x, i = li / NC, c = li % NC;
-            const float4 a = r.v[grp][x];
+            const float4 a = __builtin_bit_cast(float4, src[x]);
             o[4 * c + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, p.p[i], o[4 * c + 0], 0, 0, 0);
             o[4 * c + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, p.p[i], o[4 * c + 1], 0, 0, 0);
             o[4 * c + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, p.p[i], o[4 * c + 2], 0, 0, 0);
@@ -309,20 +289,35 @@ template <int D> struct Wave<float, D> {
     }
 };
 
+// Dynamic LDS of the partial kernel: the query operands, later overlaid by WAVES/2
+// reduction slots of one wave's O accumulators each, then per-wave (max, sum) rows.
+template <typename KV, int D, int WAVES> struct PartialLds {
+    using W = Wave<KV, D>;
+    static constexpr size_t kSlotBytes = (size_t)W::NACC * 64 * 16;
+    static constexpr size_t kQBytes = (size_t)W::QLDS_U4 * 16;
+    static constexpr size_t kRedBytes = kSlotBytes * (WAVES / 2);
+    static constexpr size_t kRegion0 = kRedBytes > kQBytes ? kRedBytes : kQBytes;
+    static constexpr size_t kBytes = kRegion0 + 2 * WAVES * 16 * sizeof(float);
+};
+
 // part_o:  [kv head][head group][split][16 heads][D]
 // part_ml: [kv head][head group][split][2][16]   (max in log2 units, then sum)
-template <typename KV, int D>
-__global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
+template <typename KV, int D, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
     const float *__restrict__ q, int hpk, int64_t kv_len, int blocks_per_split, float qscale,
     float *__restrict__ part_o, float *__restrict__ part_ml) {
     using W = Wave<KV, D>;
+    using L = PartialLds<KV, D, WAVES>;
     constexpr int NACC = W::NACC;
     constexpr int NG = W::NG;
-    __shared__ uint4 qlds[W::QLDS_U4];
-    __shared__ float sm[kWaves][16];
-    __shared__ float sl[kWaves][16];
-    __shared__ f32x4 red[2][NACC][64];
+    constexpr int G = W::G;
+    constexpr int NITEM = 2 * NG;  // a block's stream: NG groups of K, then NG groups of V
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    uint4 *qlds = reinterpret_cast<uint4 *>(lds_raw);
+    f32x4 *red = reinterpret_cast<f32x4 *>(lds_raw);  // [WAVES/2][NACC][64], after the main loop
+    float *sm = reinterpret_cast<float *>(lds_raw + L::kRegion0);  // [WAVES][16]
+    float *sl = sm + WAVES * 16;                                   // [WAVES][16]
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -336,15 +331,15 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     int64_t b1 = b0 + blocks_per_split;
     if (b1 > nblk) b1 = nblk;
 
-    // The first block's loads go out before anything else; the query conversion
-    // below overlaps their latency.
-    typename W::Regs r;
+    // Stream item t of a block is K group t (t < NG) or V group t-NG; item t lives in
+    // buf[t & 1].  The first two items go out before anything else; the query
+    // conversion below overlaps their latency.
+    uint4 buf[2][G];
     int64_t b = b0 + wave;
     if (b < b1) {
-#pragma unroll
-        for (int x = 0; x < NG; x++) W::load_k(r, x, kplane, b, lane);
-#pragma unroll
-        for (int x = 0; x < NG; x++) W::load_v(r, x, vplane, b, lane);
+        W::load_group(buf[0], kplane, b, 0, lane);
+        if (NG > 1) W::load_group(buf[1], kplane, b, 1, lane);
+        else W::load_group(buf[1], vplane, b, 0, lane);
     }
     W::prep_q(qlds, q, kvh, hg, hpk, qscale);
     __syncthreads();
@@ -354,81 +349,86 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     for (int a = 0; a < NACC; a++) o[a] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = neg_inf(), l_run = 0.f;
 
-    for (; b < b1; b += kWaves) {
-        const int64_t bn = b + kWaves;
+    for (; b < b1; b += WAVES) {
+        const int64_t bn = b + WAVES;
         const bool more = bn < b1;
         typename W::Scores sc;
+        typename W::Probs p;
         W::zero_scores(sc);
 #pragma unroll
-        for (int x = 0; x < NG; x++) {
-            W::consume_k(r, x, qlds, lane, sc);
-            if (more) W::load_k(r, x, kplane, bn, lane);
-        }
-        typename W::Probs p;
-        const float alpha = W::softmax(sc, b, kv_len, g, m_run, l_run, p);
-        if (__any(alpha != 1.0f)) {  // the running max moved: rescale what has been accumulated
+        for (int t = 0; t < NITEM; t++) {
+            if (t == NG) {
+                const float alpha = W::softmax(sc, b, kv_len, g, m_run, l_run, p);
+                if (__any(alpha != 1.0f)) {  // the running max moved: rescale what has been accumulated
 #pragma unroll
-            for (int a = 0; a < NACC; a++) {
-                o[a][0] *= alpha; o[a][1] *= alpha; o[a][2] *= alpha; o[a][3] *= alpha;
+                    for (int a = 0; a < NACC; a++) {
+                        o[a][0] *= alpha; o[a][1] *= alpha; o[a][2] *= alpha; o[a][3] *= alpha;
+                    }
+                }
             }
-        }
-#pragma unroll
-        for (int x = 0; x < NG; x++) {
-            W::consume_v(r, x, p, o);
-            if (more) W::load_v(r, x, vplane, bn, lane);
+            if (t < NG) W::consume_k(buf[t & 1], t, qlds, lane, sc);
+            else W::consume_v(buf[t & 1], t - NG, p, o);
+            // refill the buffer just consumed with the item two ahead in the stream
+            const int t2 = t + 2;
+            if (t2 < NITEM) {
+                if (t2 < NG) W::load_group(buf[t & 1], kplane, b, t2, lane);
+                else W::load_group(buf[t & 1], vplane, b, t2 - NG, lane);
+            } else if (more) {
+                const int t3 = t2 - NITEM;
+                if (t3 < NG) W::load_group(buf[t & 1], kplane, bn, t3, lane);
+                else W::load_group(buf[t & 1], vplane, bn, t3 - NG, lane);
+            }
         }
     }
     l_run += lane_xor(l_run, 16);
     l_run += lane_xor(l_run, 32);
 
-    // ---- merge the four waves ------------------------------------------------
-    if (g == 0) sm[wave][n] = m_run;
-    __syncthreads();
-    float M = sm[0][n];
+    // ---- merge the waves ---------------------------------------------------------
+    if (g == 0) sm[wave * 16 + n] = m_run;
+    __syncthreads();  // also: every wave is done reading the query operands
+    float M = sm[n];
 #pragma unroll
-    for (int x = 1; x < kWaves; x++) M = fmaxf(M, sm[x][n]);
+    for (int x = 1; x < WAVES; x++) M = fmaxf(M, sm[x * 16 + n]);
     const float f = (m_run == neg_inf()) ? 0.f : fast_exp2(m_run - M);
     l_run *= f;
 #pragma unroll
     for (int a = 0; a < NACC; a++) {
         o[a][0] *= f; o[a][1] *= f; o[a][2] *= f; o[a][3] *= f;
     }
-    if (g == 0) sl[wave][n] = l_run;
-    if (wave >= 2) {
+    if (g == 0) sl[wave * 16 + n] = l_run;
 #pragma unroll
-        for (int a = 0; a < NACC; a++) red[wave - 2][a][lane] = o[a];
-    }
-    __syncthreads();
-    if (wave < 2) {
+    for (int half = WAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
 #pragma unroll
-        for (int a = 0; a < NACC; a++) {
-            const f32x4 t = red[wave][a][lane];
-            o[a][0] += t[0]; o[a][1] += t[1]; o[a][2] += t[2]; o[a][3] += t[3];
+            for (int a = 0; a < NACC; a++) red[((wave - half) * NACC + a) * 64 + lane] = o[a];
         }
-    }
-    __syncthreads();
-    if (wave == 1) {
+        __syncthreads();
+        if (wave < half) {
 #pragma unroll
-        for (int a = 0; a < NACC; a++) red[0][a][lane] = o[a];
+            for (int a = 0; a < NACC; a++) {
+                const f32x4 t = red[(wave * NACC + a) * 64 + lane];
+                o[a][0] += t[0]; o[a][1] += t[1]; o[a][2] += t[2]; o[a][3] += t[3];
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (wave == 0) {
-#pragma unroll
-        for (int a = 0; a < NACC; a++) {
-            const f32x4 t = red[0][a][lane];
-            o[a][0] += t[0]; o[a][1] += t[1]; o[a][2] += t[2]; o[a][3] += t[3];
-        }
         const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
         W::store_o(part_o + (pid * 16 + n) * D, g, o);
         if (g == 0) {
+            float lsum = 0.f;
+#pragma unroll
+            for (int x = 0; x < WAVES; x++) lsum += sl[x * 16 + n];
             part_ml[pid * 32 + n] = M;
-            part_ml[pid * 32 + 16 + n] = sl[0][n] + sl[1][n] + sl[2][n] + sl[3][n];
+            part_ml[pid * 32 + 16 + n] = lsum;
         }
     }
 }
 
 // grid (Hq, D/64), 256 threads: 16 lanes x float4 cover 64 outputs of one split's row,
-// 16 such rows per pass.
+// 16 such rows per pass.  Each thread's partial rows are requested before the weights
+// are known, so the kernel pays one memory round trip.
+static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
@@ -439,11 +439,28 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const int kvh = h / hpk, hin = h % hpk, hg = hin / 16, n = hin % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
     const int dl = tid & 15, sg = tid >> 4;  // 16 float4 lanes x 16 split lanes
     const int d0 = blockIdx.y * 64 + dl * 4;
+
+    float4 rows[kMergeRows];
+#pragma unroll
+    for (int r = 0; r < kMergeRows; r++) {
+        const int s = sg + 16 * r;
+        rows[r] = (s < nsplit) ? *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0)
+                               : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    const float gt_in = (tid < 64) ? gate[(size_t)h * D + blockIdx.y * 64 + tid] : 0.f;
+
+    // every thread sees (max, sum) of up to 4 splits; nsplit <= kMaxSplits = 4 * 256
+    float ms[4], ls[4];
     float m = neg_inf();
-    for (int s = tid; s < nsplit; s += 256) m = fmaxf(m, part_ml[(pid0 + s) * 32 + n]);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int s = tid + 256 * r;
+        ms[r] = (s < nsplit) ? part_ml[(pid0 + s) * 32 + n] : neg_inf();
+        ls[r] = (s < nsplit) ? part_ml[(pid0 + s) * 32 + 16 + n] : 0.f;
+        m = fmaxf(m, ms[r]);
+    }
 #pragma unroll
     for (int x = 1; x < 64; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
     if (lane == 0) redf[wave] = m;
@@ -451,11 +468,12 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float M = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
     __syncthreads();
     float den = 0.f;
-    for (int s = tid; s < nsplit; s += 256) {
-        const float ms = part_ml[(pid0 + s) * 32 + n];
-        const float ws = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
-        wsh[s] = ws;
-        den += ws * part_ml[(pid0 + s) * 32 + 16 + n];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int s = tid + 256 * r;
+        const float ws = (ms[r] == neg_inf()) ? 0.f : fast_exp2(ms[r] - M);
+        if (s < nsplit) wsh[s] = ws;
+        den += ws * ls[r];
     }
 #pragma unroll
     for (int x = 1; x < 64; x <<= 1) den += __shfl_xor(den, x, 64);
@@ -464,7 +482,13 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     den = redf[0] + redf[1] + redf[2] + redf[3];
 
     float4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s = sg; s < nsplit; s += 16) {
+#pragma unroll
+    for (int r = 0; r < kMergeRows; r++) {
+        const int s = sg + 16 * r;
+        const float w = (s < nsplit) ? wsh[s] : 0.f;
+        acc.x += w * rows[r].x; acc.y += w * rows[r].y; acc.z += w * rows[r].z; acc.w += w * rows[r].w;
+    }
+    for (int s = sg + 16 * kMergeRows; s < nsplit; s += 16) {
         const float w = wsh[s];
         const float4 v = *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0);
         acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
@@ -478,7 +502,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
 #pragma unroll
         for (int x = 0; x < 16; x++) t += ((const float *)&acc4[x][ql])[qc];
         const int d = blockIdx.y * 64 + tid;
-        const float gt = 1.0f / (1.0f + expf(-gate[(size_t)h * D + d]));
+        const float gt = 1.0f / (1.0f + expf(-gt_in));
         out[(size_t)h * D + d] = (t / den) * gt;
     }
 }
@@ -555,26 +579,34 @@ bool sdpa_shape_supported(int kv_dtype, int head_dim) {
 
 static int blk_of(int kv_dtype) { return kv_dtype == MFA_KV_BF16 ? 32 : 16; }
 
-int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced) {
-    (void)D;
+// Partition of the cache's position blocks over workgroups.  Workgroups have 8 waves
+// (one block in flight per wave) when that still leaves one workgroup per CU, else 4.
+struct SplitPlan {
+    int splits;
+    int waves;
+    int64_t bps;  // blocks per split
+};
+
+static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int64_t kv_len, int num_cus, int forced) {
     const int hpk = Hq / Hkv;
     const int nhg = (hpk + 15) / 16;
     const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
     int64_t target = forced > 0 ? forced : (num_cus / (Hkv * nhg));
     if (target < 1) target = 1;
     if (target > kMaxSplits) target = kMaxSplits;
-    int64_t bps = (nblk + target - 1) / target;
-    if (forced <= 0 && bps < kWaves) bps = kWaves;  // at least one block per wave
-    if (bps < 1) bps = 1;
-    int64_t ns = (nblk + bps - 1) / bps;
-    if (ns < 1) ns = 1;
-    return (int)ns;
+    SplitPlan p;
+    p.bps = (nblk + target - 1) / target;
+    if (p.bps < 1) p.bps = 1;
+    p.waves = p.bps >= 8 ? 8 : 4;
+    if (forced <= 0 && p.bps < p.waves) p.bps = p.waves;  // at least one block per wave
+    p.splits = (int)((nblk + p.bps - 1) / p.bps);
+    if (p.splits < 1) p.splits = 1;
+    return p;
 }
 
-static int64_t bps_for(int kv_dtype, int64_t kv_len, int splits) {
-    const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
-    int64_t bps = (nblk + splits - 1) / splits;
-    return bps < 1 ? 1 : bps;
+int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced) {
+    (void)D;
+    return plan_splits(kv_dtype, Hq, Hkv, kv_len, num_cus, forced).splits;
 }
 
 size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits) {
@@ -586,13 +618,31 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits) {
     return (size_t)Hkv * nhg * splits * 32;
 }
 
-template <typename KV, int D>
-static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
-                           size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
-                           float qscale, float *po, float *pml) {
-    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D>), grid, dim3(kWaves * 64), 0, stream,
+template <typename KV, int D, int WAVES>
+static int launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
+                          size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
+                          float qscale, float *po, float *pml) {
+    constexpr size_t lds = PartialLds<KV, D, WAVES>::kBytes;
+    static bool attr_set = false;  // more than 64 KiB of dynamic LDS has to be allowed once per kernel
+    if (lds > 48 * 1024 && !attr_set) {
+        MFA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_partial_kernel<KV, D, WAVES>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES>), grid, dim3(WAVES * 64), lds, stream,
                        (const KV *)k, (const KV *)v, plane_elems, q, hpk, kv_len, bps, qscale, po,
                        pml);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
+}
+
+template <typename KV, int D>
+static int launch_partial_w(int waves, hipStream_t stream, dim3 grid, const void *k, const void *v,
+                            size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
+                            float qscale, float *po, float *pml) {
+    if (waves == 8)
+        return launch_partial<KV, D, 8>(stream, grid, k, v, plane_elems, q, hpk, kv_len, bps, qscale, po, pml);
+    return launch_partial<KV, D, 4>(stream, grid, k, v, plane_elems, q, hpk, kv_len, bps, qscale, po, pml);
 }
 
 int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
@@ -604,22 +654,20 @@ int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D,
     if (kv_len <= 0) return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld)", (long long)kv_len);
     const int hpk = Hq / Hkv;
     const int nhg = (hpk + 15) / 16;
-    int splits = sdpa_pick_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced_splits);
+    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, kv_len, num_cus, forced_splits);
     // never exceed the workspace
-    while (splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, splits) > ws.part_o_elems ||
-                          sdpa_workspace_ml_elems(Hq, Hkv, splits) > ws.part_ml_elems))
-        splits = (splits + 1) / 2;
-    if (sdpa_workspace_o_elems(Hq, Hkv, D, splits) > ws.part_o_elems)
+    while (plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits) > ws.part_o_elems ||
+                               sdpa_workspace_ml_elems(Hq, Hkv, plan.splits) > ws.part_ml_elems))
+        plan = plan_splits(kv_dtype, Hq, Hkv, kv_len, num_cus, (plan.splits + 1) / 2);
+    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits) > ws.part_o_elems)
         return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small");
-    const int64_t bps = bps_for(kv_dtype, kv_len, splits);
-    const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
-    splits = (int)((nblk + bps - 1) / bps);
     // scores are produced in log2 units: q is pre-multiplied by (1/sqrt(D)) * log2(e)
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
-    dim3 grid(splits, nhg, Hkv);
-#define MFA_LAUNCH(KV, DD)                                                                      \
-    launch_partial<KV, DD>(stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, kv_len, (int)bps, \
-                           qscale, ws.part_o, ws.part_ml)
+    dim3 grid(plan.splits, nhg, Hkv);
+    int rc;
+#define MFA_LAUNCH(KV, DD)                                                                        \
+    rc = launch_partial_w<KV, DD>(plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, \
+                                  kv_len, (int)plan.bps, qscale, ws.part_o, ws.part_ml)
     if (kv_dtype == MFA_KV_BF16) {
         if (D == 64) MFA_LAUNCH(uint16_t, 64);
         else if (D == 128) MFA_LAUNCH(uint16_t, 128);
@@ -630,10 +678,10 @@ int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D,
         else MFA_LAUNCH(float, 256);
     }
 #undef MFA_LAUNCH
-    MFA_HIP(hipGetLastError());
+    MFA_TRY(rc);
     if (partial_only) return MFA_OK;
     hipLaunchKernelGGL(sdpa_merge_kernel, dim3(Hq, D / 64), dim3(256), 0, stream, ws.part_o,
-                       ws.part_ml, splits, hpk, nhg, D, gate, out);
+                       ws.part_ml, plan.splits, hpk, nhg, D, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

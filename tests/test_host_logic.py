@@ -23,7 +23,7 @@ def test_tiling_is_a_bijection_on_every_block(dtype, blk, D, is_v):
 def test_tiling_matches_the_decode_kernels_operand_order():
     """bf16: lane (row m = lane%16, group g = lane/16) of load `li` in a block reads 8
     consecutive elements at li*512 + lane*8; they must be channels 8*(4s+g)..+7 of position
-    16*sub + m for K (li = sub*D/32 + s), and for V the 8 positions
+    16*sub + m for K (li = 2*s + sub), and for V the 8 positions
     {4g..4g+3, 16+4g..16+4g+3} of channel 16*dt + m (li = dt)."""
     lib = ffi.load()
     D = 256
@@ -31,7 +31,7 @@ def test_tiling_matches_the_decode_kernels_operand_order():
         for lane in (0, 17, 38, 63):
             m, g = lane % 16, lane // 16
             base = li * 512 + lane * 8
-            sub, s = li // (D // 32), li % (D // 32)
+            s, sub = li // 2, li % 2
             for e in range(8):
                 assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, 16 * sub + m, 8 * (4 * s + g) + e, D) == base + e
                 pos = 16 * (e // 4) + 4 * g + e % 4
