@@ -60,7 +60,7 @@ __host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 //   V: [dt = x/16][g = (p%16)/4][m = x%16][e = 4*(p/16) + p%4]
 // f32, block of 16 positions:
 //   K: [chunk = x/4][row = p][e = x%4]
-//   V: [i = p%4][c = x/64][g = p/4][m = (x%64)/4][j = x%4]
+//   V: [dt = x/16][g = p/4][m = x%16][j = p%4]
 template <typename T> struct KvTile;
 
 template <> struct KvTile<uint16_t> {
@@ -89,9 +89,7 @@ template <> struct KvTile<float> {
     __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
         const int64_t blk = pos / 16;
         const int p = (int)(pos % 16);
-        const int i = p % 4, g = p / 4;
-        const int c = x / 64, m = (x % 64) / 4, j = x % 4;
-        return blk * 16 * D + ((((int64_t)i * (D / 64) + c) * 4 + g) * 16 + m) * 4 + j;
+        return blk * 16 * D + ((((int64_t)(x / 16)) * 4 + p / 4) * 16 + (x % 16)) * 4 + (p % 4);
     }
 };
 

@@ -36,17 +36,16 @@ def test_tiling_matches_the_decode_kernels_operand_order():
                 assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 0, 16 * sub + m, 8 * (4 * s + g) + e, D) == base + e
                 pos = 16 * (e // 4) + 4 * g + e % 4
                 assert lib.mfa_debug_kv_offset(ffi.KV_BF16, 1, pos, 16 * li + m, D) == base + e
-    # f32: K load s holds channels 4*(4s+g)..+3 of position m; V load li = i*NC + c holds
-    # channels 64c + 4m .. +3 of position 4g + i
+    # f32: K load s holds channels 4*(4s+g)..+3 of position m; V load dt holds positions
+    # 4g .. 4g+3 of channel 16 dt + m
     D = 128
     for li in (0, 3, 7):
         for lane in (0, 21, 63):
             m, g = lane % 16, lane // 16
             base = li * 256 + lane * 4
-            i, c = li // (D // 64), li % (D // 64)
             for j in range(4):
                 assert lib.mfa_debug_kv_offset(ffi.KV_F32, 0, m, 4 * (4 * li + g) + j, D) == base + j
-                assert lib.mfa_debug_kv_offset(ffi.KV_F32, 1, 4 * g + i, 64 * c + 4 * m + j, D) == base + j
+                assert lib.mfa_debug_kv_offset(ffi.KV_F32, 1, 4 * g + j, 16 * li + m, D) == base + j
 
 
 def test_tiling_rejects_bad_arguments():
