@@ -219,11 +219,45 @@ static int truncate_full(Ctx *c, FullLayer &f, int32_t new_len) {
     return MFA_OK;
 }
 
-static int sdpa_decode_dev(Ctx *c, FullLayer *f, const float *q, const float *gate, float *out) {
+// The split-K workspace is sized for decode at create time; a prompt chunk has n_tok times
+// the rows and grows it on first use.
+static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len) {
+    const mfa_config &g = c->cfg;
+    int splits = sdpa_pick_splits(g.kv_dtype, g.num_attn_heads, g.num_kv_heads, g.head_dim, kv_len,
+                                  c->num_cus, c->forced_splits);
+    if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
+    const size_t need_o = sdpa_workspace_o_elems(g.num_attn_heads, g.num_kv_heads, g.head_dim, splits, n_tok);
+    const size_t need_ml = sdpa_workspace_ml_elems(g.num_attn_heads, g.num_kv_heads, splits, n_tok);
+    if (need_o <= c->part_o_elems && need_ml <= c->part_ml_elems) return MFA_OK;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    if (need_o > c->part_o_elems) {
+        if (c->part_o) MFA_HIP(hipFree(c->part_o));
+        c->part_o = nullptr;
+        c->part_o_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->part_o, need_o * sizeof(float)));
+        c->part_o_elems = need_o;
+    }
+    if (need_ml > c->part_ml_elems) {
+        if (c->part_ml) MFA_HIP(hipFree(c->part_ml));
+        c->part_ml = nullptr;
+        c->part_ml_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->part_ml, need_ml * sizeof(float)));
+        c->part_ml_elems = need_ml;
+    }
+    return MFA_OK;
+}
+
+// n_tok tokens whose K/V rows are already in the cache (the last n_tok positions).
+static int sdpa_dev(Ctx *c, FullLayer *f, int n_tok, const float *q, const float *gate, float *out) {
     if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
-    return launch_sdpa_decode(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
-                              c->cfg.head_dim, f->len, c->plane_elems, f->k, f->v, q, gate, out,
-                              workspace(c), c->num_cus, c->forced_splits, c->partial_only);
+    if (n_tok > 1) MFA_TRY(ensure_workspace(c, n_tok, f->len));
+    return launch_sdpa(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
+                       c->cfg.head_dim, n_tok, f->len, c->plane_elems, f->k, f->v, q, gate, out,
+                       workspace(c), c->num_cus, c->forced_splits, c->partial_only);
+}
+
+static int sdpa_decode_dev(Ctx *c, FullLayer *f, const float *q, const float *gate, float *out) {
+    return sdpa_dev(c, f, 1, q, gate, out);
 }
 
 static int kv_append_dev(Ctx *c, FullLayer *f, const float *k, const float *v, int64_t rows) {
@@ -309,8 +343,8 @@ static int sdpa_stateless(int kv_dtype, int32_t kv_len, int32_t Hq, int32_t Hkv,
     MFA_TRY(pml.alloc(ws.part_ml_elems * 4));
     ws.part_o = po.as<float>();
     ws.part_ml = pml.as<float>();
-    MFA_TRY(launch_sdpa_decode(nullptr, kv_dtype, Hq, Hkv, D, kv_len, plane, kt.p, vt.p,
-                               dq.as<float>(), dg.as<float>(), dout.as<float>(), ws, ncu, 0));
+    MFA_TRY(launch_sdpa(nullptr, kv_dtype, Hq, Hkv, D, 1, kv_len, plane, kt.p, vt.p, dq.as<float>(),
+                        dg.as<float>(), dout.as<float>(), ws, ncu, 0));
     return dout.download(out, qd * 4);
 }
 
@@ -445,12 +479,9 @@ int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_
     if ((int64_t)f->len + T > c->cfg.kv_capacity)
         return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %d > capacity %d", f->len, T,
                     c->cfg.kv_capacity);
-    const size_t qd = (size_t)c->q_dim(), kvd = (size_t)c->kv_dim();
-    for (int t = 0; t < T; t++) {
-        MFA_TRY(kv_append_dev(c, f, k_dev + t * kvd, v_dev + t * kvd, 1));
-        MFA_TRY(sdpa_decode_dev(c, f, q_dev + t * qd, q_gate_dev + t * qd, out_dev + t * qd));
-    }
-    return MFA_OK;
+    // append the whole chunk, then one causal pass: row t sees positions [0, len0 + t]
+    MFA_TRY(kv_append_dev(c, f, k_dev, v_dev, T));
+    return sdpa_dev(c, f, T, q_dev, q_gate_dev, out_dev);
 }
 
 int mfa_prefill_attn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q, const float *q_gate,

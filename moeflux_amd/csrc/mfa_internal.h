@@ -166,12 +166,14 @@ struct SdpaWorkspace {
 bool sdpa_shape_supported(int kv_dtype, int head_dim);
 // Number of splits the launcher will use (for workspace sizing pass kv_len = capacity).
 int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced);
-size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits);
-size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits);
-int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
-                       size_t plane_elems, const void *k_tiled, const void *v_tiled,
-                       const float *q, const float *gate, float *out, const SdpaWorkspace &ws,
-                       int num_cus, int forced_splits, int partial_only = 0);
+size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok = 1);
+size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok = 1);
+// n_tok query tokens (q, gate, out: [n_tok, Hq*D]) against a cache of kv_len positions that
+// already holds them; token t attends to positions [0, kv_len - n_tok + t].  n_tok = 1 is decode.
+int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
+                size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
+                const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
+                int forced_splits, int partial_only = 0);
 // Scatter `n_rows` row-major rows ([n_rows, Hkv*D], f32 or bf16 source) into the
 // tiled planes starting at position pos0.
 int launch_kv_scatter(hipStream_t stream, int kv_dtype, int src_is_bf16, int Hkv, int D,

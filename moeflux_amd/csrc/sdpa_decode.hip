@@ -70,6 +70,28 @@ __device__ inline uint4 stream_load(const uint4 *p) {
     return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p)));
 }
 
+// The 16 rows a workgroup serves.  Row rr = 16*hg + n of kv head kvh is query head
+// rr % hpk (within the kv head's group) of token rr / hpk: one token in decode, the
+// n_tok tokens of a prompt chunk otherwise.  Token t sees positions [0, kv_len0 + t].
+struct RowGroup {
+    int kvh, hg, hpk, Hq, n_tok;
+    int64_t kv_len0;  // cache length before the first of the n_tok tokens was appended
+    __device__ bool valid(int n) const { return hg * 16 + n < n_tok * hpk; }
+    __device__ size_t q_row(int n) const {
+        const int rr = hg * 16 + n;
+        return (size_t)(rr / hpk) * Hq + kvh * hpk + rr % hpk;
+    }
+    __device__ int64_t limit(int n) const { return valid(n) ? kv_len0 + (hg * 16 + n) / hpk + 1 : 0; }
+    // smallest and largest limit among the valid rows (uniform over the workgroup)
+    __device__ int64_t limit_min() const { return kv_len0 + (hg * 16) / hpk + 1; }
+    __device__ int64_t limit_max() const {
+        int last = hg * 16 + 15;
+        if (last > n_tok * hpk - 1) last = n_tok * hpk - 1;
+        return kv_len0 + last / hpk + 1;
+    }
+    __device__ bool full() const { return hg * 16 + 15 < n_tok * hpk; }
+};
+
 // Per-dtype pieces of the kernel.  Common shape: a block's K is NLOAD 1 KiB loads,
 // its V is NACC = D/16 1 KiB loads, load `dt` of V being the 16-wide output tile dt.
 template <typename KV, int D> struct Wave;
@@ -87,14 +109,13 @@ template <int D> struct Wave<uint16_t, D> {
     static constexpr int QRAW_F4 = 2;            // float4 loads per slot
     static constexpr int P_U4 = 2;               // hi and lo probability operands per lane
 
-    __device__ static void load_q_slot(float4 (&raw)[QRAW_F4], const float *q, int slot, int kvh,
-                                       int hg, int hpk) {
+    __device__ static void load_q_slot(float4 (&raw)[QRAW_F4], const float *q, int slot,
+                                       const RowGroup &rows) {
         const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
-        const int hin = hg * 16 + n;
         const float4 z = {0.f, 0.f, 0.f, 0.f};
         raw[0] = raw[1] = z;
-        if (hin < hpk) {
-            const float *p = q + (size_t)(kvh * hpk + hin) * D + 8 * (4 * s + g);
+        if (rows.valid(n)) {
+            const float *p = q + rows.q_row(n) * D + 8 * (4 * s + g);
             raw[0] = *(const float4 *)p;
             raw[1] = *(const float4 *)(p + 4);
         }
@@ -172,12 +193,11 @@ template <int D> struct Wave<float, D> {
     static constexpr int QRAW_F4 = 1;
     static constexpr int P_U4 = 1;
 
-    __device__ static void load_q_slot(float4 (&raw)[QRAW_F4], const float *q, int slot, int kvh,
-                                       int hg, int hpk) {
+    __device__ static void load_q_slot(float4 (&raw)[QRAW_F4], const float *q, int slot,
+                                       const RowGroup &rows) {
         const int s = slot >> 6, lane = slot & 63, n = lane & 15, g = lane >> 4;
-        const int hin = hg * 16 + n;
         raw[0] = float4{0.f, 0.f, 0.f, 0.f};
-        if (hin < hpk) raw[0] = *(const float4 *)(q + (size_t)(kvh * hpk + hin) * D + 4 * (4 * s + g));
+        if (rows.valid(n)) raw[0] = *(const float4 *)(q + rows.q_row(n) * D + 4 * (4 * s + g));
     }
     // Query operands in LDS: [k-step][lane] float4; lane (n, g) holds q[n][4(4s+g) .. +3].
     __device__ static void store_q_slot(uint4 *qlds, const float4 (&raw)[QRAW_F4], int slot, float qscale) {
@@ -230,8 +250,8 @@ template <int D> struct Wave<float, D> {
 template <typename KV, int D, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
-    const float *__restrict__ q, int hpk, int64_t kv_len, int blocks_per_split, float qscale,
-    float *__restrict__ part_o, float *__restrict__ part_ml) {
+    const float *__restrict__ q, int hpk, int Hq, int n_tok, int64_t kv_len0,
+    int blocks_per_split, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml) {
     using W = Wave<KV, D>;
     constexpr int NACC = W::NACC;
     constexpr int TPW = NACC / WAVES;  // output tiles owned by one wave
@@ -252,10 +272,22 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const int64_t blk_elems = (int64_t)W::BLK * D;
     const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
     const KV *vplane = v_tiled + (size_t)kvh * plane_elems;
-    const int64_t nblk = (kv_len + W::BLK - 1) / W::BLK;
+    const RowGroup rows{kvh, hg, hpk, Hq, n_tok, kv_len0};
+    const int64_t limit = rows.limit(n);          // this lane's row sees positions [0, limit)
+    const int64_t limit_min = rows.limit_min();   // below it no row of the group is masked
+    const bool all_rows = rows.full();
+    const int64_t nblk = (rows.limit_max() + W::BLK - 1) / W::BLK;
     const int64_t b0 = (int64_t)split * blocks_per_split;
     int64_t b1 = b0 + blocks_per_split;
     if (b1 > nblk) b1 = nblk;
+    const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
+    if (b0 >= b1) {  // a split that lies wholly beyond what this group's rows may see
+        if (wave == 0 && g == 0) {
+            part_ml[pid * 32 + n] = neg_inf();
+            part_ml[pid * 32 + 16 + n] = 0.f;
+        }
+        return;
+    }
 
     // ---- requests, in the order they are needed (loads return in order) ---------
     // Every load below is unconditional (indices are clamped instead), so that the
@@ -266,7 +298,7 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     for (int i = 0; i < NQ; i++) {
         int slot = threadIdx.x + i * WAVES * 64;
         if (slot >= W::QSLOTS) slot = W::QSLOTS - 1;
-        W::load_q_slot(qraw[i], q, slot, kvh, hg, hpk);
+        W::load_q_slot(qraw[i], q, slot, rows);
     }
     // A CU returns load data in request order across its waves: hold the bulk requests
     // back until every wave's query request is queued, or a late wave's query would
@@ -320,10 +352,10 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
             W::unpack(sc, x);
         }
         if (more) load_k(sb + WAVES);  // the K registers are free again
-        if (!have || (blk + 1) * W::BLK > kv_len) {  // the cache's last block is ragged; a clamped re-read is void
+        if (!have || !all_rows || (blk + 1) * W::BLK > limit_min) {  // a block some row must not see in full
 #pragma unroll
             for (int e = 0; e < NX; e++)
-                if (!have || W::pos_of(blk, g, e) >= kv_len) x[e] = neg_inf();
+                if (!have || W::pos_of(blk, g, e) >= limit) x[e] = neg_inf();
         }
 #pragma unroll
         for (int e = 0; e < NX; e++) m_loc = fmaxf(m_loc, x[e]);
@@ -333,15 +365,17 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
         __syncthreads();
         float m_new = m_run;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) m_new = fmaxf(m_new, sm[w][n]);  // finite: block sb is never empty
-        const float alpha = fast_exp2(m_run - m_new);
+        for (int w = 0; w < WAVES; w++) m_new = fmaxf(m_new, sm[w][n]);
+        // a row that has seen nothing yet (its limit lies further on, or it is padding) keeps -inf
+        const float m_ref = (m_new == neg_inf()) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run - m_ref);
         m_run = m_new;
         float psum = 0.f;
         {
             float e[NX];
 #pragma unroll
             for (int i = 0; i < NX; i++) {
-                e[i] = fast_exp2(x[i] - m_new);  // 0 for masked positions
+                e[i] = fast_exp2(x[i] - m_ref);  // 0 for masked positions
                 psum += e[i];
             }
             uint4 p[W::P_U4];
@@ -379,7 +413,6 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     l_run += lane_xor(l_run, 16);
     l_run += lane_xor(l_run, 32);
     if (g == 0) sl[wave][n] = l_run;
-    const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
     float *row = part_o + (pid * 16 + n) * D;
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
@@ -403,12 +436,13 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
 static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
-    int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
+    int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
     __shared__ float wsh[kMaxSplits];
     __shared__ float redf[4];
     __shared__ float4 acc4[16][16];
-    const int h = blockIdx.x;
-    const int kvh = h / hpk, hin = h % hpk, hg = hin / 16, n = hin % 16;
+    // blockIdx.x = token * Hq + head; its row in the kv head's row list is token*hpk + head%hpk
+    const int h = blockIdx.x % Hq, tok = blockIdx.x / Hq;
+    const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int dl = tid & 15, sg = tid >> 4;  // 16 float4 lanes x 16 split lanes
@@ -429,7 +463,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
         rows[r] = (s < nsplit) ? *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0)
                                : float4{0.f, 0.f, 0.f, 0.f};
     }
-    const float gt_in = (tid < 64) ? gate[(size_t)h * D + blockIdx.y * 64 + tid] : 0.f;
+    const float gt_in = (tid < 64) ? gate[(size_t)blockIdx.x * D + blockIdx.y * 64 + tid] : 0.f;
 
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
 #pragma unroll
@@ -474,7 +508,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
         for (int x = 0; x < 16; x++) t += ((const float *)&acc4[x][ql])[qc];
         const int d = blockIdx.y * 64 + tid;
         const float gt = 1.0f / (1.0f + expf(-gt_in));
-        out[(size_t)h * D + d] = (t / den) * gt;
+        out[(size_t)blockIdx.x * D + d] = (t / den) * gt;
     }
 }
 
@@ -487,22 +521,24 @@ static int blk_of(int kv_dtype) { return kv_dtype == MFA_KV_BF16 ? 32 : 16; }
 
 // Partition of the cache's position blocks over workgroups.  A workgroup has 8 waves
 // (super-blocks of 8 blocks) when that still gives every CU a workgroup, else 4;
-// head_dim 64 has only 4 output tiles, hence 4 waves.
+// head_dim 64 has only 4 output tiles, hence 4 waves.  n_tok > 1 (a prompt chunk)
+// multiplies the row groups, which already fill the machine, so the cache is split less.
 struct SplitPlan {
     int splits;
     int waves;
+    int nhg;      // 16-row groups per kv head
     int64_t bps;  // blocks per split
 };
 
-static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus,
-                             int forced) {
+static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
+                             int num_cus, int forced) {
     const int hpk = Hq / Hkv;
-    const int nhg = (hpk + 15) / 16;
+    SplitPlan p;
+    p.nhg = (int)(((int64_t)n_tok * hpk + 15) / 16);
     const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
-    int64_t target = forced > 0 ? forced : (num_cus / (Hkv * nhg));
+    int64_t target = forced > 0 ? forced : (num_cus / ((int64_t)Hkv * p.nhg));
     if (target < 1) target = 1;
     if (target > kMaxSplits) target = kMaxSplits;
-    SplitPlan p;
     p.bps = (nblk + target - 1) / target;
     if (p.bps < 1) p.bps = 1;
     p.waves = (p.bps >= 8 && D >= 128) ? 8 : 4;
@@ -513,62 +549,70 @@ static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_le
 }
 
 int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced) {
-    return plan_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced).splits;
+    return plan_splits(kv_dtype, Hq, Hkv, D, 1, kv_len, num_cus, forced).splits;
 }
 
-size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits) {
-    const int nhg = (Hq / Hkv + 15) / 16;
+size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok) {
+    const int64_t nhg = ((int64_t)n_tok * (Hq / Hkv) + 15) / 16;
     return (size_t)Hkv * nhg * splits * 16 * D;
 }
-size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits) {
-    const int nhg = (Hq / Hkv + 15) / 16;
+size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok) {
+    const int64_t nhg = ((int64_t)n_tok * (Hq / Hkv) + 15) / 16;
     return (size_t)Hkv * nhg * splits * 32;
 }
 
 template <typename KV, int D, int WAVES>
 static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
-                           size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
-                           float qscale, float *po, float *pml) {
+                           size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
+                           int64_t kv_len0, int bps, float qscale, float *po, float *pml) {
     hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES>), grid, dim3(WAVES * 64), 0, stream,
-                       (const KV *)k, (const KV *)v, plane_elems, q, hpk, kv_len, bps, qscale, po,
-                       pml);
+                       (const KV *)k, (const KV *)v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
+                       qscale, po, pml);
 }
 
 template <typename KV, int D>
 static void launch_partial_w(int waves, hipStream_t stream, dim3 grid, const void *k, const void *v,
-                             size_t plane_elems, const float *q, int hpk, int64_t kv_len, int bps,
-                             float qscale, float *po, float *pml) {
+                             size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
+                             int64_t kv_len0, int bps, float qscale, float *po, float *pml) {
     if constexpr (D >= 128) {
         if (waves == 8) {
-            launch_partial<KV, D, 8>(stream, grid, k, v, plane_elems, q, hpk, kv_len, bps, qscale, po, pml);
+            launch_partial<KV, D, 8>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
+                                     qscale, po, pml);
             return;
         }
     }
-    launch_partial<KV, D, 4>(stream, grid, k, v, plane_elems, q, hpk, kv_len, bps, qscale, po, pml);
+    launch_partial<KV, D, 4>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, qscale,
+                             po, pml);
 }
 
-int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len,
-                       size_t plane_elems, const void *k_tiled, const void *v_tiled,
-                       const float *q, const float *gate, float *out, const SdpaWorkspace &ws,
-                       int num_cus, int forced_splits, int partial_only) {
+// n_tok query tokens against a cache of kv_len positions that already holds them: token t
+// (t = 0 is position kv_len - n_tok) attends to positions [0, kv_len - n_tok + t].
+// q, gate, out: [n_tok, Hq*D].  n_tok = 1 is decode.
+int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
+                size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
+                const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
+                int forced_splits, int partial_only) {
     if (!sdpa_shape_supported(kv_dtype, D))
         return fail(MFA_ERR_SHAPE, "sdpa: head_dim %d / kv dtype %d not supported", D, kv_dtype);
-    if (kv_len <= 0) return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld)", (long long)kv_len);
+    if (n_tok <= 0 || kv_len < n_tok)
+        return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld for %d tokens)", (long long)kv_len, n_tok);
     const int hpk = Hq / Hkv;
-    const int nhg = (hpk + 15) / 16;
-    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced_splits);
+    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
     // never exceed the workspace
-    while (plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits) > ws.part_o_elems ||
-                               sdpa_workspace_ml_elems(Hq, Hkv, plan.splits) > ws.part_ml_elems))
-        plan = plan_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, (plan.splits + 1) / 2);
-    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits) > ws.part_o_elems)
+    while (plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
+                               sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems))
+        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
+    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
+        sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems)
         return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small");
+    if (plan.nhg > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
     // scores are produced in log2 units: q is pre-multiplied by (1/sqrt(D)) * log2(e)
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
-    dim3 grid(plan.splits, nhg, Hkv);
-#define MFA_LAUNCH(KV, DD)                                                                         \
-    launch_partial_w<KV, DD>(plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, kv_len, \
-                             (int)plan.bps, qscale, ws.part_o, ws.part_ml)
+    const int64_t kv_len0 = kv_len - n_tok;
+    dim3 grid(plan.splits, plan.nhg, Hkv);
+#define MFA_LAUNCH(KV, DD)                                                                          \
+    launch_partial_w<KV, DD>(plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, Hq, n_tok, \
+                             kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml)
     if (kv_dtype == MFA_KV_BF16) {
         if (D == 64) MFA_LAUNCH(uint16_t, 64);
         else if (D == 128) MFA_LAUNCH(uint16_t, 128);
@@ -581,8 +625,8 @@ int launch_sdpa_decode(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D,
 #undef MFA_LAUNCH
     MFA_HIP(hipGetLastError());
     if (partial_only) return MFA_OK;
-    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(Hq, D / 64), dim3(256), 0, stream, ws.part_o,
-                       ws.part_ml, plan.splits, hpk, nhg, D, gate, out);
+    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, ws.part_o,
+                       ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

@@ -1,0 +1,179 @@
+"""GPU tests of the stateful surface: prompt chunks, the whole-stack sweep, and the
+state operations (memory_clear / memory_seq_rm / pos_max, export / import), through
+the C ABI, against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from tests.util import TOL_F32, GdnCase, rel_err, sdpa_random_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _full_ctx(mfa, Hq, Hkv, d, cap, bf16=False, layers=1):
+    from moeflux_amd import Config
+    return mfa.Ctx(Config(num_layers=layers, full_attn_interval=1, num_attn_heads=Hq,
+                          num_kv_heads=Hkv, head_dim=d, kv_capacity=cap, kv_dtype=1 if bf16 else 0))
+
+
+@pytest.mark.parametrize("T,L0", [(1, 0), (5, 0), (33, 0), (17, 40), (64, 31)])
+def test_prefill_attn_equals_the_token_loop(mfa, oracle, T, L0):
+    """A chunk of T tokens after L0 cached positions: row t is decode with kv_len = L0+t+1
+    (riir/mod.rs:1196-1214)."""
+    Hq, Hkv, d = 32, 4, 128
+    rng = np.random.default_rng(T * 100 + L0)
+    k = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    v = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+    with _full_ctx(mfa, Hq, Hkv, d, 128) as c:
+        if L0:
+            c.kv_import(0, k[:L0], v[:L0])
+        out = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+        assert c.kv_len(0) == L0 + T
+        ke, ve = c.kv_export(0)
+    assert rel_err(out, ref) <= TOL_F32
+    for t in range(T):
+        assert rel_err(out[t], ref[t]) <= 5e-5, t
+    assert np.array_equal(ke, k) and np.array_equal(ve, v)
+
+
+def test_prefill_attn_bf16_chunk_of_512(mfa, oracle):
+    """BASELINE config 4, attention half: 512 tokens, 32 Q / 4 KV heads, d=128, bf16 values,
+    from an empty cache."""
+    Hq, Hkv, d, T = 32, 4, 128, 512
+    rng = np.random.default_rng(0xC0FFEE + 4)
+    kb = oracle.f32_to_bf16(rng.standard_normal((T, Hkv * d)).astype(np.float32))
+    vb = oracle.f32_to_bf16(rng.standard_normal((T, Hkv * d)).astype(np.float32))
+    k, v = oracle.bf16_to_f32(kb), oracle.bf16_to_f32(vb)
+    q = oracle.bf16_to_f32(oracle.f32_to_bf16((rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)))
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    ref = oracle.prefill_attn(T, 0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+    with _full_ctx(mfa, Hq, Hkv, d, 512, bf16=True) as c:
+        out = c.prefill_attn(0, q, g, k, v)
+    assert rel_err(out, ref) <= 1e-2      # the stated tolerance of the bf16 path
+    assert rel_err(out, ref) <= 1e-4
+
+
+def test_token_sweep_equals_independent_calls(mfa, oracle):
+    """One token's attention launches over a hybrid stack (every 4th layer full attention,
+    variants.rs:258-264) equal the per-layer calls."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    NL, Hq, Hkv, d, L = 8, 32, 2, 256, 200
+    case = GdnCase(9, 16, 32, 128, 128)
+    cfg = Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=256, kv_dtype=1)
+    rng = np.random.default_rng(77)
+    n_full, n_lin = 2, 6
+    qs, gs, ks, vs = [], [], [], []
+    with mfa.Ctx(cfg) as c:
+        lib = c.lib
+        for i in range(NL):
+            if cfg.is_full(i):
+                q, g, k, v = sdpa_random_inputs(300 + i, Hq, Hkv, d, L, bf16=True)
+                c.kv_import(i, k, v)
+                qs.append(q); gs.append(g); ks.append(k); vs.append(v)
+            else:
+                c.set_linear_weights(i, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+        lin_states = [((rng.standard_normal(3 * case.C)).astype(np.float32),
+                       (rng.standard_normal(32 * 128 * 128) * 0.02).astype(np.float32)) for _ in range(n_lin)]
+        lin_idx = [i for i in range(NL) if not cfg.is_full(i)]
+        for (cs, ss), i in zip(lin_states, lin_idx):
+            c.linear_state_import(i, cs, ss)
+        x = rng.standard_normal((n_lin, case.C)).astype(np.float32)
+        z = rng.standard_normal((n_lin, 32 * 128)).astype(np.float32)
+        al = rng.standard_normal((n_lin, 32)).astype(np.float32)
+        be = rng.standard_normal((n_lin, 32)).astype(np.float32)
+        dq, dg = DeviceArray.from_host(np.array(qs)), DeviceArray.from_host(np.array(gs))
+        dfo = DeviceArray((n_full, Hq * d), np.float32, zero=True)
+        dx, dz, da, db = (DeviceArray.from_host(a) for a in (x, z, al, be))
+        dlo = DeviceArray((n_lin, 32 * 128), np.float32, zero=True)
+        rc = lib.mfa_token_sweep_dev(c.h, dq.ptr, dg.ptr, dfo.ptr, dx.ptr, dz.ptr, da.ptr, db.ptr, dlo.ptr)
+        assert rc == 0, ffi.last_error()
+        c.sync()
+        fo, lo = dfo.to_host(), dlo.to_host()
+        new_states = [c.linear_state_export(i) for i in lin_idx]
+    for j in range(n_full):
+        assert rel_err(fo[j], oracle.sdpa(L, Hq, Hkv, d, qs[j], gs[j], ks[j], vs[j])) <= 1e-4
+    for j in range(n_lin):
+        ro, rc_, rs = oracle.gdn_step(16, 32, 128, 128, 4, 1e-6, case.conv_w, case.a_log, case.dt_bias,
+                                      case.norm_w, x[j], z[j], al[j], be[j], *lin_states[j])
+        assert rel_err(lo[j], ro) <= TOL_F32
+        assert np.array_equal(new_states[j][0].reshape(-1), rc_)
+        assert rel_err(new_states[j][1], rs) <= TOL_F32
+
+
+def test_state_operations_follow_the_reference(mfa, oracle):
+    """memory_seq_rm keeps [0, p0) of every KV cache and zero-fills the rest, resets every
+    DeltaNet layer (state.rs:431-455); memory_clear empties everything; pos_max is the
+    largest KV length (state.rs:457-473)."""
+    from moeflux_amd import Config
+    Hq, Hkv, d = 8, 2, 64
+    case = GdnCase(4, 2, 4, 64, 64)
+    cfg = Config(num_layers=4, full_attn_interval=2, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=64, linear_num_k_heads=2, linear_num_v_heads=4, linear_key_dim=64,
+                 linear_value_dim=64)
+    q, g, k, v = sdpa_random_inputs(5, Hq, Hkv, d, 40)
+    with mfa.Ctx(cfg) as c:
+        assert c.memory_seq_pos_max() == 0
+        for layer in (1, 3):
+            c.kv_import(layer, k[:40 if layer == 1 else 25], v[:40 if layer == 1 else 25])
+        for layer in (0, 2):
+            c.set_linear_weights(layer, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+            c.linear_state_import(layer, case.conv_state, case.ssm_state)
+            c.gdn_step(layer, case.qkv[0], case.z[0], case.alpha[0], case.beta[0])
+        assert c.memory_seq_pos_max() == 40
+        c.memory_seq_rm(30, -1)
+        assert c.kv_len(1) == 30 and c.kv_len(3) == 25 and c.memory_seq_pos_max() == 30
+        assert rel_err(c.sdpa_decode(1, q, g), oracle.sdpa(30, Hq, Hkv, d, q, g, k, v)) <= TOL_F32
+        for layer in (0, 2):
+            cs, ss = c.linear_state_export(layer)
+            assert not cs.any() and not ss.any()
+        # the dropped rows are zero: re-append one row and export
+        c.kv_append(1, k[30], v[30])
+        ke, ve = c.kv_export(1)
+        assert np.array_equal(ke, k[:31]) and np.array_equal(ve, v[:31])
+        # a DeltaNet layer restarted from zero behaves like a fresh one
+        o = c.gdn_step(0, case.qkv[0], case.z[0], case.alpha[0], case.beta[0])
+        ro, _, _ = oracle.gdn_step(2, 4, 64, 64, 4, 1e-6, case.conv_w, case.a_log, case.dt_bias, case.norm_w,
+                                   case.qkv[0], case.z[0], case.alpha[0], case.beta[0],
+                                   np.zeros_like(case.conv_state), np.zeros_like(case.ssm_state))
+        assert rel_err(o, ro) <= TOL_F32
+        c.memory_seq_rm(100, -1)          # past the end: no-op for KV, DeltaNet still reset
+        assert c.kv_len(1) == 31
+        c.memory_clear()
+        assert c.memory_seq_pos_max() == 0 and c.kv_len(1) == 0 and c.kv_len(3) == 0
+
+
+def test_error_paths_leave_the_context_usable(mfa, oracle):
+    from moeflux_amd import Config, MfaError, ffi
+    Hq, Hkv, d = 8, 2, 64
+    cfg = Config(num_layers=2, full_attn_interval=2, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=3, linear_num_k_heads=2, linear_num_v_heads=4, linear_key_dim=64,
+                 linear_value_dim=64)
+    q, g, k, v = sdpa_random_inputs(6, Hq, Hkv, d, 4)
+    with mfa.Ctx(cfg) as c:
+        with pytest.raises(MfaError) as e:
+            c.sdpa_decode(1, q, g)                       # empty cache: kv_len <= 0 (sdpa.rs:71)
+        assert e.value.code == ffi.ERR_INVALID
+        with pytest.raises(MfaError) as e:
+            c.sdpa_decode(0, q, g)                       # layer 0 is a DeltaNet layer
+        assert e.value.code == ffi.ERR_LAYER
+        with pytest.raises(MfaError) as e:
+            c.kv_len(7)
+        assert e.value.code == ffi.ERR_LAYER
+        for p in range(3):
+            c.kv_append(1, k[p], v[p])
+        with pytest.raises(MfaError) as e:
+            c.kv_append(1, k[3], v[3])                   # overflow (full_attn_forward.rs:283-288)
+        assert e.value.code == ffi.ERR_OVERFLOW
+        case = GdnCase(4, 2, 4, 64, 64)
+        with pytest.raises(MfaError) as e:
+            c.gdn_step(0, case.qkv[0], case.z[0], case.alpha[0], case.beta[0])   # weights not set
+        assert e.value.code == ffi.ERR_INVALID
+        assert c.lib.mfa_sdpa_decode(c.h, 1, None, None, None) == ffi.ERR_INVALID
+        # still works after all of that
+        assert rel_err(c.sdpa_decode(1, q, g), oracle.sdpa(3, Hq, Hkv, d, q, g, k, v)) <= TOL_F32
