@@ -25,6 +25,8 @@ ARCH = "gfx950"
 # -packed-fp32-ops off: v_pk_*_f32 forms are not to be generated for this target pool.
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+    # a*b+c fuses only where the source says fmaf(), as in the CPU oracle and the reference
+    "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
     "-I", os.path.join(ROOT, "include"), "-I", CSRC,

@@ -93,6 +93,7 @@ static void destroy(Ctx *c) {
     if (c->part_o) (void)hipFree(c->part_o);
     if (c->part_ml) (void)hipFree(c->part_ml);
     if (c->stage) (void)hipFree(c->stage);
+    if (c->gdn_scratch) (void)hipFree(c->gdn_scratch);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -523,10 +524,24 @@ int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv
     if (!qkv_in_dev || !z_dev || !alpha_dev || !beta_dev || !out_dev)
         return fail(MFA_ERR_INVALID, "NULL argument");
     if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
-    const size_t C = (size_t)c->conv_dim(), tv = (size_t)c->v_total(), Hv = (size_t)c->cfg.linear_num_v_heads;
-    for (int t = 0; t < T; t++)
-        MFA_TRY(gdn_step_dev(c, l, qkv_in_dev + t * C, z_dev + t * tv, alpha_dev + t * Hv,
-                             beta_dev + t * Hv, out_dev + t * tv));
+    if (T == 1) return gdn_step_dev(c, l, qkv_in_dev, z_dev, alpha_dev, beta_dev, out_dev);
+    if (!l->w.set) return fail(MFA_ERR_INVALID, "linear layer weights not set (mfa_set_linear_weights)");
+    const mfa_config &g = c->cfg;
+    const size_t need = gdn_chunk_scratch_elems(g.linear_num_k_heads, g.linear_num_v_heads,
+                                                g.linear_key_dim, g.linear_value_dim, T);
+    if (need > c->gdn_scratch_elems) {
+        MFA_HIP(hipStreamSynchronize(c->stream));
+        if (c->gdn_scratch) MFA_HIP(hipFree(c->gdn_scratch));
+        c->gdn_scratch = nullptr;
+        c->gdn_scratch_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->gdn_scratch, need * sizeof(float)));
+        c->gdn_scratch_elems = need;
+    }
+    MFA_TRY(launch_gdn_chunk(c->stream, g.linear_num_k_heads, g.linear_num_v_heads, g.linear_key_dim,
+                             g.linear_value_dim, g.conv_kernel_size, g.rms_norm_eps, T, l->w,
+                             l->conv_ring, l->step, l->ssm, qkv_in_dev, z_dev, alpha_dev, beta_dev,
+                             c->gdn_scratch, out_dev));
+    l->step += T;
     return MFA_OK;
 }
 

@@ -14,51 +14,9 @@
 //
 // The remaining kernels in this file are one-launch twins of the five
 // reference kernels for per-kernel parity tests.
-#include "mfa_internal.h"
+#include "gdn_device.h"
 
 namespace mfa {
-
-__device__ inline float silu_f(float x) { return x / (1.0f + expf(-x)); }
-
-template <int W> __device__ inline float group_sum(float v) {
-#pragma unroll
-    for (int m = 1; m < W; m <<= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-
-// Delta-rule update of one state row held by 8 lanes (lane j owns floats
-// 32*i + 4*j .. +3 for i < DK/32).  Follows the operation order of
-// crates/moeflux/src/riir/linear_attn.rs:383-410: decay, kv_mem, delta,
-// rank-1 update, read-out from the updated row.
-template <int DK>
-__device__ inline float delta_row(float4 (&s)[DK / 32], const float4 (&kk)[DK / 32],
-                                  const float4 (&qq)[DK / 32], float g, float beta, float v) {
-    constexpr int NI = DK / 32;
-    float kv = 0.f;
-#pragma unroll
-    for (int i = 0; i < NI; i++) {
-        s[i].x *= g; s[i].y *= g; s[i].z *= g; s[i].w *= g;
-        kv = fmaf(s[i].x, kk[i].x, kv);
-        kv = fmaf(s[i].y, kk[i].y, kv);
-        kv = fmaf(s[i].z, kk[i].z, kv);
-        kv = fmaf(s[i].w, kk[i].w, kv);
-    }
-    kv = group_sum<8>(kv);
-    const float delta = (v - kv) * beta;
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < NI; i++) {
-        s[i].x = fmaf(kk[i].x, delta, s[i].x);
-        s[i].y = fmaf(kk[i].y, delta, s[i].y);
-        s[i].z = fmaf(kk[i].z, delta, s[i].z);
-        s[i].w = fmaf(kk[i].w, delta, s[i].w);
-        o = fmaf(s[i].x, qq[i].x, o);
-        o = fmaf(s[i].y, qq[i].y, o);
-        o = fmaf(s[i].z, qq[i].z, o);
-        o = fmaf(s[i].w, qq[i].w, o);
-    }
-    return group_sum<8>(o);
-}
 
 // grid: Hv workgroups of DV*8 threads.
 template <int DK, int DV>

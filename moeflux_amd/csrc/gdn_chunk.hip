@@ -1,0 +1,197 @@
+// A chunk of T prompt tokens through one Gated-DeltaNet layer.
+//
+// The reference has no batched prefill: eval_prompt is a token loop
+// (crates/moeflux/src/riir/mod.rs:1196-1214), every token running the
+// five-kernel chain of crates/moeflux/src/riir/linear_attn_forward.rs:607-664
+// and re-reading and re-writing the [dv, dk] state.  Here the chunk is three
+// launches whose results are those of the loop, token for token:
+//
+//   gdn_chunk_pre_kernel    everything that does not depend on the state, for all T
+//                           tokens at once: conv + SiLU, per-head q/k norm, decay, beta.
+//   gdn_chunk_recur_kernel  one workgroup per value head keeps the state in registers
+//                           (8 lanes per row) across the whole chunk; the state is read
+//                           once and written once per chunk instead of once per token.
+//                           k^, q^, v, g, beta of a slab of tokens are staged in LDS.
+//   gdn_chunk_post_kernel   gated RMS norm for all (token, head) pairs, and the conv
+//                           history ring advanced by T inputs.
+#include "gdn_device.h"
+
+namespace mfa {
+
+static constexpr int kSlab = 32;  // tokens staged in LDS at a time
+
+// grid (T, Hk + ceil(Hv*DV / 256) + 1), 256 threads.
+//   y <  Hk            : q and k channels of k-head y (conv, SiLU, norm, scaling)
+//   Hk <= y < Hk + nvb : 256 v channels each (conv, SiLU)
+//   y == Hk + nvb      : decay and beta of every value head
+template <int DK>
+__global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
+    int Hk, int Hv, int DV, int K, int64_t step, const uint16_t *__restrict__ conv_w,
+    const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
+    const float *__restrict__ ring, const float *__restrict__ qkv, const float *__restrict__ alpha,
+    const float *__restrict__ beta, float *__restrict__ qn, float *__restrict__ kn,
+    float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg) {
+    static_assert(2 * DK <= 256, "one workgroup covers a k-head's q and k channels");
+    __shared__ float s_part[4];
+    const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x;
+    const int C = 2 * Hk * DK + Hv * DV;
+    const int nvb = (Hv * DV + 255) / 256;
+    if (y < Hk) {
+        // threads [0, DK) are q channels, [DK, 2DK) are k channels of this head
+        const bool act = tid < 2 * DK, is_q = tid < DK;
+        float c = 0.f;
+        if (act) {
+            const int ch = is_q ? y * DK + tid : Hk * DK + y * DK + (tid - DK);
+            c = conv_silu(ring, qkv, conv_w, C, K, step, t, ch);
+        }
+        const float ws = group_sum<64>(act ? c * c : 0.f);
+        if ((tid & 63) == 0) s_part[tid >> 6] = ws;
+        __syncthreads();
+        if (act) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < DK / 64; w++) sum += s_part[(is_q ? 0 : DK / 64) + w];
+            // infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2, k *= 1/sqrt(dk)
+            const float inv_rms = 1.0f / sqrtf(sum / (float)DK + 1e-6f);
+            const float inv_scale = 1.0f / sqrtf((float)DK);
+            float v = c * inv_rms;
+            v *= is_q ? inv_scale * inv_scale : inv_scale;
+            if (is_q) qn[((size_t)t * Hk + y) * DK + tid] = v;
+            else kn[((size_t)t * Hk + y) * DK + (tid - DK)] = v;
+        }
+    } else if (y < Hk + nvb) {
+        const int i = (y - Hk) * 256 + tid;
+        if (i < Hv * DV) vv[(size_t)t * Hv * DV + i] = conv_silu(ring, qkv, conv_w, C, K, step, t, 2 * Hk * DK + i);
+    } else {
+        for (int h = tid; h < Hv; h += 256) {
+            // shaders.metal:1321-1326
+            const float a_cap = expf(a_log[h]);
+            const float sp = logf(1.0f + expf(alpha[(size_t)t * Hv + h] + bf16_bits_to_f32(dt_bias[h])));
+            gd[(size_t)t * Hv + h] = expf(-a_cap * sp);
+            bg[(size_t)t * Hv + h] = 1.0f / (1.0f + expf(-beta[(size_t)t * Hv + h]));
+        }
+    }
+}
+
+// grid Hv, DV*8 threads.  o_raw [T, Hv*DV] receives the un-normalised read-outs.
+template <int DK, int DV>
+__global__ __launch_bounds__(DV * 8) void gdn_chunk_recur_kernel(
+    int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ kn,
+    const float *__restrict__ vv, const float *__restrict__ gd, const float *__restrict__ bg,
+    float *__restrict__ ssm, float *__restrict__ o_raw) {
+    constexpr int NI = DK / 32;
+    constexpr int NT = DV * 8;
+    __shared__ __align__(16) float s_k[kSlab][DK];
+    __shared__ __align__(16) float s_q[kSlab][DK];
+    __shared__ float s_v[kSlab][DV];
+    __shared__ float s_g[kSlab], s_b[kSlab];
+    const int tid = threadIdx.x, vh = blockIdx.x, kh = vh / (Hv / Hk);
+    const int r = tid >> 3, j = tid & 7;
+    float *srow = ssm + ((size_t)vh * DV + r) * DK + 4 * j;
+    float4 s[NI];
+#pragma unroll
+    for (int i = 0; i < NI; i++) s[i] = *(const float4 *)(srow + 32 * i);
+
+    for (int t0 = 0; t0 < T; t0 += kSlab) {
+        const int nt = (T - t0 < kSlab) ? T - t0 : kSlab;
+        __syncthreads();  // the previous slab has been consumed
+        for (int i = tid; i < nt * DK; i += NT) {
+            const int tt = i / DK, x = i % DK;
+            s_k[tt][x] = kn[((size_t)(t0 + tt) * Hk + kh) * DK + x];
+            s_q[tt][x] = qn[((size_t)(t0 + tt) * Hk + kh) * DK + x];
+        }
+        for (int i = tid; i < nt * DV; i += NT) {
+            const int tt = i / DV, x = i % DV;
+            s_v[tt][x] = vv[((size_t)(t0 + tt) * Hv + vh) * DV + x];
+        }
+        if (tid < nt) {
+            s_g[tid] = gd[(size_t)(t0 + tid) * Hv + vh];
+            s_b[tid] = bg[(size_t)(t0 + tid) * Hv + vh];
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; tt++) {
+            float4 kk[NI], qq[NI];
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                kk[i] = *(const float4 *)(&s_k[tt][32 * i + 4 * j]);
+                qq[i] = *(const float4 *)(&s_q[tt][32 * i + 4 * j]);
+            }
+            const float o = delta_row<DK>(s, kk, qq, s_g[tt], s_b[tt], s_v[tt][r]);
+            if (j == 0) o_raw[((size_t)(t0 + tt) * Hv + vh) * DV + r] = o;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; i++) *(float4 *)(srow + 32 * i) = s[i];
+}
+
+// grid (T, Hv) for the gated norm (shaders.metal:1337-1370) plus, at x == T, blocks that
+// advance the conv ring: input number s lives in slot s % K, so the last min(T, K)
+// inputs of the chunk overwrite their slots.
+__global__ __launch_bounds__(128) void gdn_chunk_post_kernel(
+    int Hv, int DV, int T, int C, int K, int64_t step, float eps, const float *__restrict__ o_raw,
+    const float *__restrict__ z, const uint16_t *__restrict__ norm_w, const float *__restrict__ qkv,
+    float *__restrict__ ring, float *__restrict__ out) {
+    __shared__ float s_part[2];
+    const int tid = threadIdx.x;
+    if ((int)blockIdx.x == T) {
+        const int first = T > K ? T - K : 0;
+        for (int t = first; t < T; t++) {
+            const int slot = (int)((step + t) % K);
+            for (int ch = blockIdx.y * 128 + tid; ch < C; ch += gridDim.y * 128)
+                ring[(size_t)slot * C + ch] = qkv[(size_t)t * C + ch];
+        }
+        return;
+    }
+    const size_t base = ((size_t)blockIdx.x * Hv + blockIdx.y) * DV;
+    float sq = 0.f;
+    for (int i = tid; i < DV; i += 128) sq += o_raw[base + i] * o_raw[base + i];
+    const float ws = group_sum<64>(sq);
+    if ((tid & 63) == 0) s_part[tid >> 6] = ws;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((s_part[0] + s_part[1]) / (float)DV + eps);
+    for (int i = tid; i < DV; i += 128)
+        out[base + i] = o_raw[base + i] * inv * bf16_bits_to_f32(norm_w[i]) * silu_f(z[base + i]);
+}
+
+size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T) {
+    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 2 * (size_t)Hv);
+}
+
+int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
+                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
+                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
+                     float *scratch, float *out) {
+    if (!gdn_shape_supported(Hk, Hv, dk, dv, K))
+        return fail(MFA_ERR_SHAPE, "gdn chunk: shape Hk=%d Hv=%d dk=%d dv=%d K=%d not supported", Hk, Hv,
+                    dk, dv, K);
+    if (T <= 0) return fail(MFA_ERR_INVALID, "gdn chunk: T must be > 0");
+    if (T > 65535) return fail(MFA_ERR_SHAPE, "gdn chunk: at most 65535 tokens per call");
+    const int C = 2 * Hk * dk + Hv * dv;
+    float *qn = scratch;
+    float *kn = qn + (size_t)T * Hk * dk;
+    float *vv = kn + (size_t)T * Hk * dk;
+    float *o_raw = vv + (size_t)T * Hv * dv;
+    float *gd = o_raw + (size_t)T * Hv * dv;
+    float *bg = gd + (size_t)T * Hv;
+    const int nvb = (Hv * dv + 255) / 256;
+    if (dk == 128) {
+        hipLaunchKernelGGL((gdn_chunk_pre_kernel<128>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
+                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
+                           vv, gd, bg);
+        hipLaunchKernelGGL((gdn_chunk_recur_kernel<128, 128>), dim3(Hv), dim3(1024), 0, s, Hk, Hv, T, qn,
+                           kn, vv, gd, bg, ssm, o_raw);
+    } else {
+        hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
+                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
+                           vv, gd, bg);
+        hipLaunchKernelGGL((gdn_chunk_recur_kernel<64, 64>), dim3(Hv), dim3(512), 0, s, Hk, Hv, T, qn, kn,
+                           vv, gd, bg, ssm, o_raw);
+    }
+    MFA_HIP(hipGetLastError());
+    hipLaunchKernelGGL(gdn_chunk_post_kernel, dim3(T + 1, Hv), dim3(128), 0, s, Hv, dv, T, C, K, step, eps,
+                       o_raw, z, w.norm_w, qkv_in, conv_ring, out);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
+}
+
+}  // namespace mfa

@@ -1,0 +1,88 @@
+// Device helpers shared by the Gated-DeltaNet kernels (gdn.hip, gdn_chunk.hip).
+#pragma once
+
+#include "mfa_internal.h"
+
+namespace mfa {
+
+__device__ inline float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+// v + (v of the lane selected by a DPP control word); no LDS round trip.
+template <int CTRL> __device__ inline float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+    return v + __builtin_bit_cast(float, t);
+}
+
+// Sum over aligned groups of W lanes, result in every lane of the group.
+// 8: quad_perm(1,0,3,2), quad_perm(2,3,0,1), row_half_mirror; 16: + row_mirror;
+// 64: the four row sums are combined through v_readlane.
+template <int W> __device__ inline float group_sum(float v) {
+    static_assert(W == 8 || W == 16 || W == 64, "group width");
+    v = dpp_add<0xB1>(v);
+    v = dpp_add<0x4E>(v);
+    v = dpp_add<0x141>(v);
+    if (W >= 16) v = dpp_add<0x140>(v);
+    if (W == 64) {
+        const int b = __builtin_bit_cast(int, v);
+        v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16)) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)) +
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    }
+    return v;
+}
+
+// Delta-rule update of one state row held by 8 lanes (lane j owns floats
+// 32*i + 4*j .. +3 for i < DK/32).  Follows the operation order of
+// crates/moeflux/src/riir/linear_attn.rs:383-410: decay, kv_mem, delta,
+// rank-1 update, read-out from the updated row.
+template <int DK>
+__device__ inline float delta_row(float4 (&s)[DK / 32], const float4 (&kk)[DK / 32],
+                                  const float4 (&qq)[DK / 32], float g, float beta, float v) {
+    constexpr int NI = DK / 32;
+    float kv = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        s[i].x *= g; s[i].y *= g; s[i].z *= g; s[i].w *= g;
+        kv = fmaf(s[i].x, kk[i].x, kv);
+        kv = fmaf(s[i].y, kk[i].y, kv);
+        kv = fmaf(s[i].z, kk[i].z, kv);
+        kv = fmaf(s[i].w, kk[i].w, kv);
+    }
+    kv = group_sum<8>(kv);
+    const float delta = (v - kv) * beta;
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        s[i].x = fmaf(kk[i].x, delta, s[i].x);
+        s[i].y = fmaf(kk[i].y, delta, s[i].y);
+        s[i].z = fmaf(kk[i].z, delta, s[i].z);
+        s[i].w = fmaf(kk[i].w, delta, s[i].w);
+        o = fmaf(s[i].x, qq[i].x, o);
+        o = fmaf(s[i].y, qq[i].y, o);
+        o = fmaf(s[i].z, qq[i].z, o);
+        o = fmaf(s[i].w, qq[i].w, o);
+    }
+    return group_sum<8>(o);
+}
+
+// Depthwise conv + SiLU of channel ch for the input numbered `step + t` of the layer
+// (crates/moeflux/src/riir/linear_attn.rs:132-154): tap k < K-1 multiplies input
+// step+t-(K-1)+k, which is row t-(K-1)+k of `chunk` when that is >= 0 and the ring slot
+// (input number mod K) of the history otherwise; tap K-1 multiplies the new input.
+__device__ inline float conv_silu(const float *__restrict__ ring, const float *__restrict__ chunk,
+                                  const uint16_t *__restrict__ w, int C, int K, int64_t step, int t,
+                                  int ch) {
+    float acc = 0.f;
+    for (int k = 0; k < K - 1; k++) {
+        const int idx = t - (K - 1) + k;
+        float x;
+        if (idx >= 0) x = chunk[(size_t)idx * C + ch];
+        else x = ring[(size_t)(((step + idx) % K + K) % K) * C + ch];
+        acc = fmaf(x, bf16_bits_to_f32(w[(size_t)ch * K + k]), acc);
+    }
+    acc = fmaf(chunk[(size_t)t * C + ch], bf16_bits_to_f32(w[(size_t)ch * K + (K - 1)]), acc);
+    return silu_f(acc);
+}
+
+}  // namespace mfa

@@ -132,6 +132,9 @@ struct Ctx {
     size_t part_o_elems = 0, part_ml_elems = 0;
     int32_t forced_splits = 0;
     int32_t partial_only = 0;
+    // scratch of the Gated-DeltaNet chunk kernels (grown on demand)
+    float *gdn_scratch = nullptr;
+    size_t gdn_scratch_elems = 0;
     // host-pointer staging
     float *stage = nullptr;
     size_t stage_elems = 0;
@@ -201,6 +204,13 @@ int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float 
                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
                     float *out);
+// gdn_chunk.hip: T tokens through one layer (three launches); scratch holds
+// gdn_chunk_scratch_elems floats.
+size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T);
+int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
+                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
+                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
+                     float *scratch, float *out);
 int launch_conv1d_step(hipStream_t s, int C, int K, float *conv_state, const float *in,
                        const uint16_t *w, float *out);
 int launch_rms_norm_qk(hipStream_t s, int Hk, int dk, float *q, float *k);

@@ -11,7 +11,7 @@ fn main() {
     let lib = out.join("libmoeflux_attn_hip.so");
     let hipcc = env::var("HIPCC").unwrap_or_else(|_| "/opt/rocm/bin/hipcc".into());
     let mut cmd = Command::new(hipcc);
-    cmd.args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"])
+    cmd.args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-ffp-contract=off"])
         .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"])
         .arg("-I").arg(root.join("include")).arg("-I").arg(&csrc);
     for f in ["api.hip", "sdpa_decode.hip", "attn_kernels.hip", "gdn.hip"] {

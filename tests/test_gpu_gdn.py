@@ -94,3 +94,43 @@ def test_gdn_kernel_hooks(mfa, oracle):
     y2 = np.concatenate([oracle.rms_norm_gated(o2[h * dv:(h + 1) * dv], z[h * dv:(h + 1) * dv],
                                                case.norm_w, 1e-6) for h in range(Hv)])
     assert rel_err(y1, y2) <= TOL_F32
+
+
+@pytest.mark.parametrize("T", [2, 3, 4, 5, 37, 100])
+def test_chunk_equals_token_loop_bit_for_bit(mfa, T):
+    """The chunk kernels do, token for token, the arithmetic of the single-step kernel
+    (riir/mod.rs:1196-1214: a prompt is a loop of steps); T below, at and above the conv
+    width exercises the history ring on both sides of the chunk boundary."""
+    case = GdnCase(40 + T, 4, 8, 128, 128, T=T)
+    with _ctx(mfa, case, num_layers=2) as c:
+        for layer in (0, 1):
+            c.linear_state_import(layer, case.conv_state, case.ssm_state)
+        chunk = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
+        loop = np.stack([c.gdn_step(1, case.qkv[t], case.z[t], case.alpha[t], case.beta[t])
+                         for t in range(T)])
+        s0, s1 = c.linear_state_export(0), c.linear_state_export(1)
+        # a further single step continues correctly from the chunk's ring and state
+        extra = GdnCase(99, 4, 8, 128, 128, T=1)
+        n0 = c.gdn_step(0, extra.qkv[0], extra.z[0], extra.alpha[0], extra.beta[0])
+        n1 = c.gdn_step(1, extra.qkv[0], extra.z[0], extra.alpha[0], extra.beta[0])
+    assert np.array_equal(chunk, loop)
+    assert np.array_equal(s0[0], s1[0]) and np.array_equal(s0[1], s1[1])
+    assert np.array_equal(n0, n1)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    assert rel_err(chunk, ref_out) <= TOL_F32
+    assert np.array_equal(s0[0].reshape(-1), ref_conv) and rel_err(s0[1], ref_ssm) <= TOL_F32
+
+
+def test_config4_gdn_chunk_of_512_from_zero_state(mfa):
+    """BASELINE config 4, DeltaNet half: 512 tokens of the config-2 shape from a zero state,
+    against 512 sequential oracle steps; outputs and the final state."""
+    case = GdnCase(0xC0FFEE + 4, 16, 32, 128, 128, T=512, zero_state=True)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case) as c:
+        out = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
+        conv, ssm = c.linear_state_export(0)
+    assert rel_err(out, ref_out) <= TOL_F32
+    worst = max(rel_err(out[t], ref_out[t]) for t in range(0, 512, 37))
+    assert worst <= 5e-5
+    assert np.array_equal(conv.reshape(-1), ref_conv)
+    assert rel_err(ssm, ref_ssm) <= TOL_F32
