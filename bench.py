@@ -31,6 +31,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per launch of the split-K partial kernel on the headline workload, from rocprofv3
+# FETCH_SIZE + WRITE_SIZE scaled by the plain copy kernel
+# (profiles/sdpa_partial_bf16_d256_c3_hbm_counters.md): 65 877 KiB read + 4 128 KiB written.
+C3_PARTIAL_TRAFFIC_BYTES = (65877 + 4128) * 1024
 
 
 def _timed(ctx, lib, fn, steps, warmup):
@@ -144,6 +148,138 @@ def bench_gdn(name, Hk, Hv, dk, dv, layers, steps, warmup, seed):
     return res
 
 
+def bench_prefill(steps, warmup, seed):
+    """BASELINE configs[3]: a 512-token prompt chunk from an empty cache / zero state —
+    causal GQA attention (32 Q / 4 KV heads, d=128, bf16 cache) and the Gated-DeltaNet
+    chunk (configs[1] shape).  Every timed call uses a fresh layer, so kv_len0 = 0."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    from tests.util import GdnCase
+    lib = ffi.load()
+    T, Hq, Hkv, d = 512, 32, 4, 128
+    n = steps + warmup
+    rng = np.random.default_rng(seed)
+    ctx = Ctx(Config(num_layers=n, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
+                     head_dim=d, kv_capacity=T, kv_dtype=ffi.KV_BF16))
+    dq = DeviceArray.from_host((rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32))
+    dg = DeviceArray.from_host(rng.standard_normal((T, Hq * d)).astype(np.float32))
+    dk = DeviceArray.from_host(rng.standard_normal((T, Hkv * d)).astype(np.float32))
+    dv = DeviceArray.from_host(rng.standard_normal((T, Hkv * d)).astype(np.float32))
+    do = DeviceArray((T, Hq * d), np.float32, zero=True)
+    layer = [0]
+
+    def step(i):
+        rc = lib.mfa_prefill_attn_dev(ctx.h, layer[0], T, dq.ptr, dg.ptr, dk.ptr, dv.ptr, do.ptr)
+        layer[0] += 1
+        if rc != 0:
+            raise RuntimeError(ffi.last_error())
+
+    wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
+    flops = 2 * 2 * Hq * (T * (T + 1) // 2) * d
+    res = {"attention_us_per_chunk": ev_ms * 1e3, "attention_causal_flop": flops,
+           "attention_tflops": flops / (ev_ms * 1e-3) / 1e12,
+           "attention_us_per_token_layer": ev_ms * 1e3 / T}
+    ctx.close()
+    for a in (dq, dg, dk, dv, do):
+        a.free()
+
+    case = GdnCase(seed, 16, 32, 128, 128, T=T, zero_state=True, plain=True)
+    layers = 8
+    ctx = Ctx(Config(num_layers=layers, full_attn_interval=layers + 1, linear_num_k_heads=16,
+                     linear_num_v_heads=32))
+    for l in range(layers):
+        ctx.set_linear_weights(l, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+    dx, dz = DeviceArray.from_host(case.qkv), DeviceArray.from_host(case.z)
+    da, db = DeviceArray.from_host(case.alpha), DeviceArray.from_host(case.beta)
+    do = DeviceArray((T, 32 * 128), np.float32, zero=True)
+
+    def gstep(i):
+        rc = lib.mfa_prefill_gdn_dev(ctx.h, i % layers, T, dx.ptr, dz.ptr, da.ptr, db.ptr, do.ptr)
+        if rc != 0:
+            raise RuntimeError(ffi.last_error())
+
+    wall_ms, ev_ms = _timed(ctx, lib, gstep, steps, warmup)
+    gflops = 7 * 128 * 128 * 32 * T
+    res.update({"deltanet_us_per_chunk": ev_ms * 1e3, "deltanet_sequential_equivalent_flop": gflops,
+                "deltanet_tflops": gflops / (ev_ms * 1e-3) / 1e12,
+                "deltanet_us_per_token_layer": ev_ms * 1e3 / T})
+    ctx.close()
+    for a in (dx, dz, da, db, do):
+        a.free()
+    return res
+
+
+def bench_sweep(steps, warmup, seed):
+    """BASELINE configs[4]: the attention launches of one token over a 48-layer hybrid stack,
+    36 Gated-DeltaNet layers (configs[1] shape) and 12 gated full-attention layers
+    (32 Q / 2 KV heads, d=256, kv_len 8192, bf16), distinct buffers per layer, in layer order
+    on one stream (mfa_token_sweep_dev)."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    from oracle import cref
+    from tests.util import GdnCase
+    lib = ffi.load()
+    NL, Hq, Hkv, d, L = 48, 32, 2, 256, 8192
+    cfg = Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=L, kv_dtype=ffi.KV_BF16, linear_num_k_heads=16, linear_num_v_heads=32)
+    ctx = Ctx(cfg)
+    rng = np.random.default_rng(seed)
+    case = GdnCase(seed, 16, 32, 128, 128, T=1, plain=True)
+    base_k = cref.f32_to_bf16(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
+    base_v = cref.f32_to_bf16(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
+    nf = nl = 0
+    for i in range(NL):
+        if cfg.is_full(i):
+            ctx.kv_import(i, base_k[8 * nf:8 * nf + L], base_v[8 * nf:8 * nf + L])
+            nf += 1
+        else:
+            ctx.set_linear_weights(i, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+            ctx.linear_state_import(i, case.conv_state,
+                                    (rng.standard_normal(32 * 128 * 128) * 0.02).astype(np.float32))
+            nl += 1
+    qd, C_, tv = Hq * d, case.C, 32 * 128
+    fq = DeviceArray.from_host((rng.standard_normal((nf, qd)) / 16).astype(np.float32))
+    fg = DeviceArray.from_host(rng.standard_normal((nf, qd)).astype(np.float32))
+    fo = DeviceArray((nf, qd), np.float32, zero=True)
+    lx = DeviceArray.from_host(rng.standard_normal((nl, C_)).astype(np.float32))
+    lz = DeviceArray.from_host(rng.standard_normal((nl, tv)).astype(np.float32))
+    la = DeviceArray.from_host(rng.standard_normal((nl, 32)).astype(np.float32))
+    lb = DeviceArray.from_host(rng.standard_normal((nl, 32)).astype(np.float32))
+    lo = DeviceArray((nl, tv), np.float32, zero=True)
+
+    def step(i):
+        rc = lib.mfa_token_sweep_dev(ctx.h, fq.ptr, fg.ptr, fo.ptr, lx.ptr, lz.ptr, la.ptr, lb.ptr, lo.ptr)
+        if rc != 0:
+            raise RuntimeError(ffi.last_error())
+
+    wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
+    alg = 36 * 4522688 + 12 * (2 * L * Hkv * d * 2 + 3 * qd * 4)
+    res = {"us_per_token_sweep": wall_ms * 1e3, "us_event": ev_ms * 1e3, "layers": NL,
+           "us_per_layer_token": wall_ms * 1e3 / NL, "algorithmic_bytes": alg,
+           "gbps": alg / (wall_ms * 1e-3) / 1e9}
+    res["pct_peak"] = 100.0 * res["gbps"] / HBM_PEAK_GBPS
+    ctx.close()
+    for a in (fq, fg, fo, lx, lz, la, lb, lo):
+        a.free()
+    return res
+
+
+def calibrate_copy(nbytes=64 << 20, reps=20):
+    """`--calibrate-copy`: launch only the plain copy kernel (nbytes read + nbytes written per
+    launch), for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    lib = ffi.load()
+    ctx = Ctx(Config(num_layers=1, full_attn_interval=2, linear_num_k_heads=1, linear_num_v_heads=1))
+    bufs = [DeviceArray((nbytes,), np.uint8, zero=True) for _ in range(8)]
+    for i in range(reps):
+        lib.mfa_debug_copy_dev(ctx.h, bufs[4 + i % 4].ptr, bufs[i % 4].ptr, nbytes)
+    ctx.sync()
+    ctx.close()
+    print(json.dumps({"copy_kernel": "plain_copy_kernel", "bytes_read_per_launch": nbytes,
+                      "bytes_written_per_launch": nbytes, "launches": reps}))
+
+
 def cpu_baseline(sample, Hq, Hkv, d, L, budget_s=12.0):
     """The CPU oracle (a port of the reference's scalar sdpa_cpu, which is what the
     reference itself runs at kv_len >= 8192), one thread, f32 cache, same inputs."""
@@ -173,11 +309,16 @@ def main():
     ap.add_argument("--layers", type=int, default=8, help="independent KV caches rotated over")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="launch only the plain copy kernel (for scaling memory counters) and exit")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path is measured on one GPU only (batch-1 decode attention on one "
               "device); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if a.calibrate_copy:
+        calibrate_copy()
+        return
 
     Hq, Hkv, d, L = 32, 2, 256, 32768
     head, sample = bench_sdpa("c3", Hq, Hkv, d, L, True, a.layers, a.steps, a.warmup, 0xC0FFEE + 3)
@@ -193,7 +334,7 @@ def main():
         "hbm_gbps": head["gbps"], "hbm_pct_peak": head["pct_peak"],
         "roofline": {"bound": "hbm", "achieved": head["gbps_partial_kernel"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": head["gbps_partial_kernel"] / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "sdpa_partial_kernel<bf16, 256>",
+                     "traffic": C3_PARTIAL_TRAFFIC_BYTES, "kernel": "sdpa_partial_kernel<bf16, 256, 8>",
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
                      "us_per_launch": head["us_partial_kernel_loop"]},
     }
@@ -208,6 +349,8 @@ def main():
         extra["c1_gqa_decode_f32_L4096"] = r
         extra["c2_gated_deltanet_step"] = bench_gdn("c2", 16, 32, 128, 128, 160, a.steps, a.warmup,
                                                     0xC0FFEE + 2)
+        extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
+        extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
         line["extra"] = extra
     print(json.dumps(line))
 

@@ -272,6 +272,11 @@ int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t num_attn_heads, int32_t n
                              int32_t head_dim, int64_t kv_len, int32_t num_cus,
                              int32_t forced_splits);
 
+/* A plain device-to-device copy kernel on the context's stream (nbytes read, nbytes
+ * written, nbytes a multiple of 16): a launch of known memory traffic, used to scale
+ * hardware memory counters when profiling.  No counterpart in the reference. */
+int mfa_debug_copy_dev(mfa_ctx *ctx, void *dst_dev, const void *src_dev, size_t nbytes);
+
 #pragma GCC visibility pop
 
 #ifdef __cplusplus

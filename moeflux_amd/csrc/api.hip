@@ -723,6 +723,12 @@ int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t Hq, int32_t Hkv, int32_t 
     return sdpa_pick_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced_splits);
 }
 
+int mfa_debug_copy_dev(mfa_ctx *ctx, void *dst_dev, const void *src_dev, size_t nbytes) {
+    Ctx *c = as_ctx(ctx);
+    if (!c || !dst_dev || !src_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    return launch_plain_copy(c->stream, dst_dev, src_dev, nbytes);
+}
+
 /* ---- timing ------------------------------------------------------------------------ */
 
 int mfa_timer_start(mfa_ctx *ctx) {

@@ -125,4 +125,20 @@ int launch_kv_zero(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plan
     return MFA_OK;
 }
 
+// Plain 16-byte-per-lane device copy (mfa_debug_copy_dev): a kernel of known traffic,
+// nbytes read and nbytes written, against which hardware memory counters are scaled.
+__global__ void plain_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes) {
+    if (nbytes % 16 != 0) return fail(MFA_ERR_INVALID, "copy size must be a multiple of 16 bytes");
+    if (nbytes == 0) return MFA_OK;
+    hipLaunchKernelGGL(plain_copy_kernel, dim3(grid_for((int64_t)(nbytes / 16), 256)), dim3(256), 0, stream,
+                       (const uint4 *)src, (uint4 *)dst, nbytes / 16);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
+}
+
 }  // namespace mfa

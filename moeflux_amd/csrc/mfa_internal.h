@@ -190,6 +190,8 @@ int launch_kv_gather(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t pl
 int launch_kv_zero(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plane_elems,
                    int64_t pos0, int64_t pos1, void *k_tiled, void *v_tiled);
 
+int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+
 // attn_kernels.hip (the four reference kernels, one launch each)
 int launch_attn_scores(hipStream_t s, int Hq, int Hkv, int D, int L, int stride, const float *q,
                        const float *k, float scale, float *scores);
