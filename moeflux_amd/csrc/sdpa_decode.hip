@@ -313,9 +313,10 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
 #pragma unroll
         for (int i = 0; i < NLOAD; i++) kreg[i] = stream_load(p + i * 64);
     };
-    auto load_v = [&](int64_t sb) {
+    // V of blocks [j0, j1) of the super-block starting at sb
+    auto load_v = [&](int64_t sb, int j0, int j1) {
 #pragma unroll
-        for (int j = 0; j < WAVES; j++) {
+        for (int j = j0; j < j1; j++) {
             int64_t blk = sb + j;
             if (blk > b1 - 1) blk = b1 - 1;
             const uint4 *p = (const uint4 *)(vplane + blk * blk_elems) + lane + (wave * TPW) * 64;
@@ -323,8 +324,12 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
             for (int t = 0; t < TPW; t++) vreg[j][t] = stream_load(p + t * 64);
         }
     };
+    // A wave issues in order, and a CU accepts only so many outstanding loads: requesting
+    // all of V here would keep the wave stuck in the issue stage long after its K has
+    // arrived.  So only kVEarly blocks of V go out now, the rest once the scores are under way.
+    constexpr int kVEarly = WAVES / 4;
     load_k(b0);
-    load_v(b0);
+    load_v(b0, 0, kVEarly);
 #pragma unroll
     for (int i = 0; i < NQ; i++) {
         const int slot = threadIdx.x + i * WAVES * 64;
@@ -339,8 +344,9 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
 
     // One super-block.  `more` is a compile-time constant at both call sites so that
     // each path has a fixed sequence of loads.
-    auto super_block = [&](int64_t sb, auto more_tag) {
+    auto super_block = [&](int64_t sb, auto more_tag, auto first_tag) {
         constexpr bool more = decltype(more_tag)::value;
+        constexpr int v_issued = decltype(first_tag)::value ? kVEarly : WAVES;  // V blocks already requested
         const int64_t blk = sb + wave;
         const bool have = blk < b1;
         // ---- phase 1: this wave's block of scores ------------------------------
@@ -351,6 +357,7 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
             W::scores(kreg, qlds, lane, sc);
             W::unpack(sc, x);
         }
+        if (v_issued < WAVES) load_v(sb, v_issued, WAVES);
         if (more) load_k(sb + WAVES);  // the K registers are free again
         if (!have || !all_rows || (blk + 1) * W::BLK > limit_min) {  // a block some row must not see in full
 #pragma unroll
@@ -401,12 +408,15 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
 #pragma unroll
             for (int t = 0; t < TPW; t++) o[t] = W::pv(vreg[j][t], p, o[t]);
         }
-        if (more) load_v(sb + WAVES);
+        if (more) load_v(sb + WAVES, 0, WAVES);
     };
-    {
-        int64_t sb = b0;
-        for (; sb + WAVES < b1; sb += WAVES) super_block(sb, std::true_type{});
-        super_block(sb, std::false_type{});
+    if (b0 + WAVES < b1) {
+        super_block(b0, std::true_type{}, std::true_type{});
+        int64_t sb = b0 + WAVES;
+        for (; sb + WAVES < b1; sb += WAVES) super_block(sb, std::true_type{}, std::false_type{});
+        super_block(sb, std::false_type{}, std::false_type{});
+    } else {
+        super_block(b0, std::false_type{}, std::true_type{});
     }
 
     // ---- one partial per workgroup -----------------------------------------------
