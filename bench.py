@@ -252,12 +252,20 @@ def bench_sweep(steps, warmup, seed):
         if rc != 0:
             raise RuntimeError(ffi.last_error())
 
-    wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
     alg = 36 * 4522688 + 12 * (2 * L * Hkv * d * 2 + 3 * qd * 4)
-    res = {"us_per_token_sweep": wall_ms * 1e3, "us_event": ev_ms * 1e3, "layers": NL,
-           "us_per_layer_token": wall_ms * 1e3 / NL, "algorithmic_bytes": alg,
-           "gbps": alg / (wall_ms * 1e-3) / 1e9}
-    res["pct_peak"] = 100.0 * res["gbps"] / HBM_PEAK_GBPS
+    res = {"layers": NL, "algorithmic_bytes": alg}
+    # "per_kind": the 36 DeltaNet layers in one launch and the 12 full-attention layers in
+    # one split-K launch + merge (all inputs of the token are known up front);
+    # "per_layer": the 48 launch chains one after another, what a caller whose layers
+    # depend on each other pays.
+    for name, per_layer in (("per_kind", 0), ("per_layer", 1)):
+        if lib.mfa_set_sweep_per_layer(ctx.h, per_layer) != 0:
+            raise RuntimeError(ffi.last_error())
+        wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
+        gbps = alg / (wall_ms * 1e-3) / 1e9
+        res[name] = {"us_per_token_sweep": wall_ms * 1e3, "us_event": ev_ms * 1e3,
+                     "us_per_layer_token": wall_ms * 1e3 / NL, "gbps": gbps,
+                     "pct_peak": 100.0 * gbps / HBM_PEAK_GBPS}
     ctx.close()
     for a in (fq, fg, fo, lx, lz, la, lb, lo):
         a.free()

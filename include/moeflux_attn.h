@@ -161,10 +161,23 @@ int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv
  * layer's slice of the inputs.  Inputs are packed per kind, in layer order:
  *   full_q, full_gate, full_out: [n_full, Hq*head_dim];
  *   lin_qkv [n_lin, C]; lin_z, lin_out [n_lin, Hv*dv]; lin_alpha, lin_beta [n_lin, Hv].
- * The KV caches are used as they stand (append first). */
+ * The KV caches are used as they stand (append first).
+ *
+ * Because all of a token's inputs are handed over at once, the layers of a kind
+ * that stand at the same position (equal kv length; equal conv ring slot) are
+ * computed by one launch over all of them; results equal the per-layer loop.
+ * A caller whose layers depend on each other (the model itself: layer i+1's
+ * projections read layer i's output) calls mfa_sdpa_decode_dev / mfa_gdn_step_dev
+ * layer by layer instead; a caller that batches independent sequences or layers
+ * uses this. */
 int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gate,
                         float *full_out, const float *lin_qkv, const float *lin_z,
                         const float *lin_alpha, const float *lin_beta, float *lin_out);
+
+/* Measurement control for mfa_token_sweep_dev: on != 0 forces one launch chain per
+ * layer (the cost a data-dependent caller sees); 0 (default) lets it launch once per
+ * kind.  No counterpart in the reference. */
+int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on);
 
 /* ---- state operations ------------------------------------------------------ */
 

@@ -78,18 +78,8 @@ static void destroy(Ctx *c) {
     if (!c) return;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    for (auto &f : c->full) {
-        if (f.k) (void)hipFree(f.k);
-        if (f.v) (void)hipFree(f.v);
-    }
-    for (auto &l : c->lin) {
-        if (l.conv_ring) (void)hipFree(l.conv_ring);
-        if (l.ssm) (void)hipFree(l.ssm);
-        if (l.w.conv_w) (void)hipFree(l.w.conv_w);
-        if (l.w.a_log) (void)hipFree(l.w.a_log);
-        if (l.w.dt_bias) (void)hipFree(l.w.dt_bias);
-        if (l.w.norm_w) (void)hipFree(l.w.norm_w);
-    }
+    for (void *p : c->slabs)
+        if (p) (void)hipFree(p);
     if (c->part_o) (void)hipFree(c->part_o);
     if (c->part_ml) (void)hipFree(c->part_ml);
     if (c->stage) (void)hipFree(c->stage);
@@ -98,6 +88,16 @@ static void destroy(Ctx *c) {
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
+}
+
+// A zero-filled device allocation owned by the context until it is destroyed.
+static int slab_alloc(Ctx *c, size_t bytes, char **out) {
+    void *p = nullptr;
+    MFA_HIP(hipMalloc(&p, bytes ? bytes : 4));
+    c->slabs.push_back(p);
+    MFA_HIP(hipMemsetAsync(p, 0, bytes, c->stream));
+    *out = (char *)p;
+    return MFA_OK;
 }
 
 static int validate(const mfa_config *cfg, bool *has_full, bool *has_lin) {
@@ -168,11 +168,15 @@ static int create(const mfa_config *cfg, Ctx **out) {
         c->cap_pad = ((int64_t)cfg->kv_capacity + blk - 1) / blk * blk;
         c->plane_elems = (size_t)c->cap_pad * cfg->head_dim;
         const size_t bytes = c->plane_elems * cfg->num_kv_heads * c->kv_elem_size();
-        for (auto &f : c->full) {
-            MFA_HIP(hipMalloc(&f.k, bytes));
-            MFA_HIP(hipMalloc(&f.v, bytes));
-            MFA_HIP(hipMemsetAsync(f.k, 0, bytes, c->stream));
-            MFA_HIP(hipMemsetAsync(f.v, 0, bytes, c->stream));
+        // One allocation for all layers' K planes and one for their V planes, layer-major:
+        // plane (layer, kv head) sits at index layer * Hkv + kv head, so a launch over all
+        // layers is a launch over nfull * Hkv kv heads.
+        char *kslab, *vslab;
+        MFA_TRY(slab_alloc(c, bytes * nfull, &kslab));
+        MFA_TRY(slab_alloc(c, bytes * nfull, &vslab));
+        for (int i = 0; i < nfull; i++) {
+            c->full[i].k = kslab + (size_t)i * bytes;
+            c->full[i].v = vslab + (size_t)i * bytes;
         }
         int splits = sdpa_pick_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
                                       cfg->head_dim, cfg->kv_capacity, c->num_cus, 0);
@@ -186,15 +190,24 @@ static int create(const mfa_config *cfg, Ctx **out) {
         const size_t C = (size_t)c->conv_dim(), K = (size_t)cfg->conv_kernel_size;
         const size_t ssm = (size_t)cfg->linear_num_v_heads * cfg->linear_value_dim * cfg->linear_key_dim;
         const int Hv = cfg->linear_num_v_heads;
-        for (auto &l : c->lin) {
-            MFA_HIP(hipMalloc((void **)&l.conv_ring, K * C * sizeof(float)));
-            MFA_HIP(hipMalloc((void **)&l.ssm, ssm * sizeof(float)));
-            MFA_HIP(hipMemsetAsync(l.conv_ring, 0, K * C * sizeof(float), c->stream));
-            MFA_HIP(hipMemsetAsync(l.ssm, 0, ssm * sizeof(float), c->stream));
-            MFA_HIP(hipMalloc((void **)&l.w.conv_w, C * K * 2));
-            MFA_HIP(hipMalloc((void **)&l.w.a_log, Hv * sizeof(float)));
-            MFA_HIP(hipMalloc((void **)&l.w.dt_bias, Hv * 2));
-            MFA_HIP(hipMalloc((void **)&l.w.norm_w, (size_t)cfg->linear_value_dim * 2));
+        // Layer-major slabs, each layer's part at a fixed stride, so that one launch can
+        // step every linear layer (the kernels offset by layer index * stride).
+        const size_t dv = (size_t)cfg->linear_value_dim;
+        char *ring, *state, *cw, *al, *dt, *nw;
+        MFA_TRY(slab_alloc(c, nlin * K * C * sizeof(float), &ring));
+        MFA_TRY(slab_alloc(c, nlin * ssm * sizeof(float), &state));
+        MFA_TRY(slab_alloc(c, nlin * C * K * 2, &cw));
+        MFA_TRY(slab_alloc(c, nlin * Hv * sizeof(float), &al));
+        MFA_TRY(slab_alloc(c, nlin * Hv * 2, &dt));
+        MFA_TRY(slab_alloc(c, nlin * dv * 2, &nw));
+        for (int i = 0; i < nlin; i++) {
+            LinearLayer &l = c->lin[i];
+            l.conv_ring = (float *)ring + (size_t)i * K * C;
+            l.ssm = (float *)state + (size_t)i * ssm;
+            l.w.conv_w = (uint16_t *)cw + (size_t)i * C * K;
+            l.w.a_log = (float *)al + (size_t)i * Hv;
+            l.w.dt_bias = (uint16_t *)dt + (size_t)i * Hv;
+            l.w.norm_w = (uint16_t *)nw + (size_t)i * dv;
         }
     }
     MFA_HIP(hipStreamSynchronize(c->stream));
@@ -222,13 +235,14 @@ static int truncate_full(Ctx *c, FullLayer &f, int32_t new_len) {
 
 // The split-K workspace is sized for decode at create time; a prompt chunk has n_tok times
 // the rows and grows it on first use.
-static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len) {
+// `layers` > 1 sizes it for one launch over that many layers (layers * Hkv kv heads).
+static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
     const mfa_config &g = c->cfg;
-    int splits = sdpa_pick_splits(g.kv_dtype, g.num_attn_heads, g.num_kv_heads, g.head_dim, kv_len,
-                                  c->num_cus, c->forced_splits);
+    const int Hq = g.num_attn_heads * layers, Hkv = g.num_kv_heads * layers;
+    int splits = sdpa_pick_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
     if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
-    const size_t need_o = sdpa_workspace_o_elems(g.num_attn_heads, g.num_kv_heads, g.head_dim, splits, n_tok);
-    const size_t need_ml = sdpa_workspace_ml_elems(g.num_attn_heads, g.num_kv_heads, splits, n_tok);
+    const size_t need_o = sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok);
+    const size_t need_ml = sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok);
     if (need_o <= c->part_o_elems && need_ml <= c->part_ml_elems) return MFA_OK;
     MFA_HIP(hipStreamSynchronize(c->stream));
     if (need_o > c->part_o_elems) {
@@ -582,7 +596,32 @@ int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gat
         return fail(MFA_ERR_INVALID, "NULL linear-attention argument");
     const size_t qd = (size_t)c->q_dim(), C = (size_t)c->conv_dim(), tv = (size_t)c->v_total(),
                  Hv = (size_t)c->cfg.linear_num_v_heads;
+    // The layers' caches, states and weights are layer-major slabs and the inputs are packed
+    // per kind, so when the layers of a kind stand at the same position the whole kind is
+    // one launch: every linear layer as a second grid dimension, every full-attention
+    // layer as n_full * Hkv kv heads.  Results are those of the layer-by-layer loop.
+    bool lin_batch = !c->sweep_per_layer && c->lin.size() > 1, full_batch = !c->sweep_per_layer && c->full.size() > 1;
+    const int64_t K = c->cfg.conv_kernel_size;
+    for (auto &l : c->lin) lin_batch = lin_batch && l.w.set && l.step % K == c->lin[0].step % K;
+    for (auto &f : c->full) full_batch = full_batch && f.len > 0 && f.len == c->full[0].len;
+    if (full_batch) {
+        const int n = (int)c->full.size();
+        MFA_TRY(ensure_workspace(c, 1, c->full[0].len, n));
+        MFA_TRY(launch_sdpa(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads * n, c->cfg.num_kv_heads * n,
+                            c->cfg.head_dim, 1, c->full[0].len, c->plane_elems, c->full[0].k, c->full[0].v,
+                            full_q, full_gate, full_out, workspace(c), c->num_cus, c->forced_splits,
+                            c->partial_only));
+    }
+    if (lin_batch) {
+        LinearLayer &l0 = c->lin[0];
+        MFA_TRY(launch_gdn_step(c->stream, c->cfg.linear_num_k_heads, c->cfg.linear_num_v_heads,
+                                c->cfg.linear_key_dim, c->cfg.linear_value_dim, c->cfg.conv_kernel_size,
+                                c->cfg.rms_norm_eps, l0.w, l0.conv_ring, l0.step, l0.ssm, lin_qkv, lin_z,
+                                lin_alpha, lin_beta, lin_out, (int)c->lin.size()));
+        for (auto &l : c->lin) l.step++;
+    }
     for (int i = 0; i < c->cfg.num_layers; i++) {
+        if (c->kind[i] == 1 ? full_batch : lin_batch) continue;
         const size_t s = (size_t)c->slot[i];
         if (c->kind[i] == 1)
             MFA_TRY(sdpa_decode_dev(c, &c->full[s], full_q + s * qd, full_gate + s * qd, full_out + s * qd));
@@ -590,6 +629,13 @@ int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gat
             MFA_TRY(gdn_step_dev(c, &c->lin[s], lin_qkv + s * C, lin_z + s * tv, lin_alpha + s * Hv,
                                  lin_beta + s * Hv, lin_out + s * tv));
     }
+    return MFA_OK;
+}
+
+int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    c->sweep_per_layer = on ? 1 : 0;
     return MFA_OK;
 }
 

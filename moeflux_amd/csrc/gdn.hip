@@ -18,8 +18,11 @@
 
 namespace mfa {
 
-// grid: Hv workgroups of DV*8 threads.
-template <int DK, int DV>
+// grid (Hv, layers): one workgroup of DV*8 threads per value head.  With more than one
+// layer every per-layer array is a layer-major slab and the packed inputs and outputs
+// are [layers, ...]: the kernel offsets each pointer by blockIdx.y strides.  KC is the conv width when it is the usual 4
+// (the taps are then requested up front, ahead of the state rows), 0 for any other width.
+template <int DK, int DV, int KC>
 __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     int Hk, int Hv, int K, float eps, const uint16_t *__restrict__ conv_w,
     const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
@@ -29,6 +32,7 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     constexpr int NI = DK / 32;
     constexpr int NT = DV * 8;
     constexpr int NWAVE = NT / 64;
+    constexpr int KT = KC > 0 ? KC : 1;
     __shared__ float s_q[DK], s_k[DK], s_v[DV], s_o[DV];
     __shared__ float s_part[NWAVE];
     __shared__ float s_gb[2];
@@ -39,8 +43,52 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     const int kh = vh / rep;
     const int C = 2 * Hk * DK + Hv * DV;
     const int r = tid >> 3, j = tid & 7;
+    {
+        const size_t ly = blockIdx.y;
+        conv_w += ly * C * K;
+        a_log += ly * Hv;
+        dt_bias += ly * Hv;
+        norm_w += ly * DV;
+        conv_ring += ly * K * C;
+        ssm += ly * Hv * DV * DK;
+        qkv_in += ly * C;
+        z += ly * Hv * DV;
+        alpha += ly * Hv;
+        beta += ly * Hv;
+        out += ly * Hv * DV;
+    }
 
-    // 1. state row loads go out first; everything below overlaps their latency.
+    // Which conv channel this thread serves: the head's q, k and v channels.
+    const bool conv_thread = tid < 2 * DK + DV;
+    int ch = 0;
+    bool owner = true;  // q/k channels are shared by `rep` value heads; one of them rolls the ring
+    if (tid < DK) { ch = kh * DK + tid; owner = (vh % rep) == 0; }
+    else if (tid < 2 * DK) { ch = Hk * DK + kh * DK + (tid - DK); owner = (vh % rep) == 0; }
+    else if (conv_thread) ch = 2 * Hk * DK + vh * DV + (tid - 2 * DK);
+
+    // 1. Requests in the order their data is needed (loads return in order): the small
+    //    operands of the conv, the gates and the output norm first, the state rows last,
+    //    so that the conv and the norms run while the state is still streaming in.
+    float x_in = 0.f, tap[KT], wt[KT];
+    if (KC > 0) {
+        x_in = qkv_in[ch];
+        const uint2 wbits = *(const uint2 *)(conv_w + (size_t)ch * 4);  // four bf16 taps
+        wt[0] = bf16_bits_to_f32((uint16_t)(wbits.x & 0xffffu));
+        if (KC > 1) wt[1 % KT] = bf16_bits_to_f32((uint16_t)(wbits.x >> 16));
+        if (KC > 2) wt[2 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y & 0xffffu));
+        if (KC > 3) wt[3 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y >> 16));
+#pragma unroll
+        for (int k = 0; k < KT - 1; k++) {
+            int sl = slot_new + 1 + k;
+            if (sl >= KC) sl -= KC;
+            tap[k] = conv_ring[(size_t)sl * C + ch];
+        }
+    }
+    const int nz = tid < DV ? tid : 0;
+    const float z_in = z[(size_t)vh * DV + nz];
+    const float nw_in = bf16_bits_to_f32(norm_w[nz]);
+    const float a_log_in = a_log[vh], alpha_in = alpha[vh], beta_in = beta[vh];
+    const float dt_in = bf16_bits_to_f32(dt_bias[vh]);
     float *srow = ssm + ((size_t)vh * DV + r) * DK + 4 * j;
     float4 s[NI];
 #pragma unroll
@@ -49,22 +97,23 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     // 2. depthwise conv + SiLU on this head's q, k and v channels
     //    (linear_attn.rs:132-154; taps oldest first, the new input is tap K-1).
     float cval = 0.f;
-    if (tid < 2 * DK + DV) {
-        int ch;
-        bool owner = true;  // q/k channels are shared by `rep` value heads; one of them rolls the ring
-        if (tid < DK) { ch = kh * DK + tid; owner = (vh % rep) == 0; }
-        else if (tid < 2 * DK) { ch = Hk * DK + kh * DK + (tid - DK); owner = (vh % rep) == 0; }
-        else ch = 2 * Hk * DK + vh * DV + (tid - 2 * DK);
-        const float x = qkv_in[ch];
+    if (conv_thread) {
         float acc = 0.f;
-        for (int k = 0; k < K - 1; k++) {
-            int sl = slot_new + 1 + k;
-            if (sl >= K) sl -= K;
-            acc = fmaf(conv_ring[(size_t)sl * C + ch], bf16_bits_to_f32(conv_w[(size_t)ch * K + k]), acc);
+        if (KC > 0) {
+#pragma unroll
+            for (int k = 0; k < KT - 1; k++) acc = fmaf(tap[k], wt[k], acc);
+            acc = fmaf(x_in, wt[KT - 1], acc);
+        } else {
+            x_in = qkv_in[ch];
+            for (int k = 0; k < K - 1; k++) {
+                int sl = slot_new + 1 + k;
+                if (sl >= K) sl -= K;
+                acc = fmaf(conv_ring[(size_t)sl * C + ch], bf16_bits_to_f32(conv_w[(size_t)ch * K + k]), acc);
+            }
+            acc = fmaf(x_in, bf16_bits_to_f32(conv_w[(size_t)ch * K + (K - 1)]), acc);
         }
-        acc = fmaf(x, bf16_bits_to_f32(conv_w[(size_t)ch * K + (K - 1)]), acc);
         cval = silu_f(acc);
-        if (owner) conv_ring[(size_t)slot_new * C + ch] = x;
+        if (owner) conv_ring[(size_t)slot_new * C + ch] = x_in;
         if (tid >= 2 * DK) s_v[tid - 2 * DK] = cval;
     }
     // 3. per-head sum of squares of q (waves [0, DK/64)) and k (waves [DK/64, 2DK/64))
@@ -75,10 +124,10 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     }
     // 4. decay and beta gate (shaders.metal:1321-1326)
     if (tid == NT - 1) {
-        const float a_cap = expf(a_log[vh]);
-        const float sp = logf(1.0f + expf(alpha[vh] + bf16_bits_to_f32(dt_bias[vh])));
+        const float a_cap = expf(a_log_in);
+        const float sp = logf(1.0f + expf(alpha_in + dt_in));
         s_gb[0] = expf(-a_cap * sp);
-        s_gb[1] = 1.0f / (1.0f + expf(-beta[vh]));
+        s_gb[1] = 1.0f / (1.0f + expf(-beta_in));
     }
     __syncthreads();
     if (tid < 2 * DK) {
@@ -119,8 +168,7 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
 #pragma unroll
             for (int w = 0; w < (DV + 63) / 64; w++) sum += s_part[w];
             const float inv_rms = 1.0f / sqrtf(sum / (float)DV + eps);
-            const float zz = z[(size_t)vh * DV + tid];
-            out[(size_t)vh * DV + tid] = x * inv_rms * bf16_bits_to_f32(norm_w[tid]) * silu_f(zz);
+            out[(size_t)vh * DV + tid] = x * inv_rms * nw_in * silu_f(z_in);
         }
     }
 }
@@ -273,19 +321,21 @@ bool gdn_shape_supported(int Hk, int Hv, int dk, int dv, int K) {
 int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps,
                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
-                    float *out) {
+                    float *out, int n_layers) {
+    if (n_layers < 1 || n_layers > 65535) return fail(MFA_ERR_INVALID, "gdn_step: bad layer count %d", n_layers);
     if (!gdn_shape_supported(Hk, Hv, dk, dv, K))
         return fail(MFA_ERR_SHAPE, "gdn_step: shape Hk=%d Hv=%d dk=%d dv=%d K=%d not supported", Hk,
                     Hv, dk, dv, K);
     const int slot_new = (int)(step % K);
-    if (dk == 128)
-        hipLaunchKernelGGL((gdn_step_kernel<128, 128>), dim3(Hv), dim3(1024), 0, s, Hk, Hv, K, eps,
-                           w.conv_w, w.a_log, w.dt_bias, w.norm_w, conv_ring, slot_new, ssm, qkv_in,
-                           z, alpha, beta, out);
-    else
-        hipLaunchKernelGGL((gdn_step_kernel<64, 64>), dim3(Hv), dim3(512), 0, s, Hk, Hv, K, eps,
-                           w.conv_w, w.a_log, w.dt_bias, w.norm_w, conv_ring, slot_new, ssm, qkv_in,
-                           z, alpha, beta, out);
+#define MFA_GDN(DKK, KCC)                                                                       \
+    hipLaunchKernelGGL((gdn_step_kernel<DKK, DKK, KCC>), dim3(Hv, n_layers), dim3(DKK * 8), 0, s, Hk, Hv, K, eps, \
+                       w.conv_w, w.a_log, w.dt_bias, w.norm_w, conv_ring, slot_new, ssm, qkv_in, z,  \
+                       alpha, beta, out)
+    if (dk == 128 && K == 4) MFA_GDN(128, 4);
+    else if (dk == 128) MFA_GDN(128, 0);
+    else if (K == 4) MFA_GDN(64, 4);
+    else MFA_GDN(64, 0);
+#undef MFA_GDN
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

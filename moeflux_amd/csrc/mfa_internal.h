@@ -124,6 +124,8 @@ struct Ctx {
     std::vector<int> slot;      // index into full / lin
     std::vector<FullLayer> full;
     std::vector<LinearLayer> lin;
+    std::vector<void *> slabs;  // device allocations behind full[] and lin[] (layer-major)
+    int32_t sweep_per_layer = 0; // 1: the token sweep launches layer by layer
     int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
     size_t plane_elems = 0;     // elements of one (layer, K|V, kv head) plane
     // split-K workspace
@@ -205,7 +207,7 @@ bool gdn_shape_supported(int Hk, int Hv, int dk, int dv, int K);
 int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps,
                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
-                    float *out);
+                    float *out, int n_layers = 1);
 // gdn_chunk.hip: T tokens through one layer (three launches); scratch holds
 // gdn_chunk_scratch_elems floats.
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T);

@@ -57,9 +57,12 @@ def test_prefill_attn_bf16_chunk_of_512(mfa, oracle):
     assert rel_err(out, ref) <= 1e-4
 
 
-def test_token_sweep_equals_independent_calls(mfa, oracle):
+@pytest.mark.parametrize("per_layer,ragged", [(0, False), (1, False), (0, True)])
+def test_token_sweep_equals_independent_calls(mfa, oracle, per_layer, ragged):
     """One token's attention launches over a hybrid stack (every 4th layer full attention,
-    variants.rs:258-264) equal the per-layer calls."""
+    variants.rs:258-264) equal the per-layer calls: launched once per layer kind, launched
+    layer by layer, and with layers at different positions (kv lengths and conv ring slots
+    differ, so the sweep has to fall back to the loop)."""
     from moeflux_amd import Config, ffi
     from moeflux_amd.hip import DeviceArray
     NL, Hq, Hkv, d, L = 8, 32, 2, 256, 200
@@ -73,7 +76,8 @@ def test_token_sweep_equals_independent_calls(mfa, oracle):
         lib = c.lib
         for i in range(NL):
             if cfg.is_full(i):
-                q, g, k, v = sdpa_random_inputs(300 + i, Hq, Hkv, d, L, bf16=True)
+                Li = L - 7 * len(qs) if ragged else L
+                q, g, k, v = sdpa_random_inputs(300 + i, Hq, Hkv, d, Li, bf16=True)
                 c.kv_import(i, k, v)
                 qs.append(q); gs.append(g); ks.append(k); vs.append(v)
             else:
@@ -91,13 +95,21 @@ def test_token_sweep_equals_independent_calls(mfa, oracle):
         dfo = DeviceArray((n_full, Hq * d), np.float32, zero=True)
         dx, dz, da, db = (DeviceArray.from_host(a) for a in (x, z, al, be))
         dlo = DeviceArray((n_lin, 32 * 128), np.float32, zero=True)
+        assert lib.mfa_set_sweep_per_layer(c.h, per_layer) == 0
+        if ragged:   # one extra token on the second linear layer: its ring slot differs
+            x0 = rng.standard_normal(case.C).astype(np.float32)
+            z0, a0, b0 = z[1] * 0.5, al[1] * 0.5, be[1] * 0.5
+            c.gdn_step(lin_idx[1], x0, z0, a0, b0)
+            _, rc0, rs0 = oracle.gdn_step(16, 32, 128, 128, 4, 1e-6, case.conv_w, case.a_log, case.dt_bias,
+                                          case.norm_w, x0, z0, a0, b0, *lin_states[1])
+            lin_states[1] = (rc0, rs0)
         rc = lib.mfa_token_sweep_dev(c.h, dq.ptr, dg.ptr, dfo.ptr, dx.ptr, dz.ptr, da.ptr, db.ptr, dlo.ptr)
         assert rc == 0, ffi.last_error()
         c.sync()
         fo, lo = dfo.to_host(), dlo.to_host()
         new_states = [c.linear_state_export(i) for i in lin_idx]
     for j in range(n_full):
-        assert rel_err(fo[j], oracle.sdpa(L, Hq, Hkv, d, qs[j], gs[j], ks[j], vs[j])) <= 1e-4
+        assert rel_err(fo[j], oracle.sdpa(len(ks[j]), Hq, Hkv, d, qs[j], gs[j], ks[j], vs[j])) <= 1e-4
     for j in range(n_lin):
         ro, rc_, rs = oracle.gdn_step(16, 32, 128, 128, 4, 1e-6, case.conv_w, case.a_log, case.dt_bias,
                                       case.norm_w, x[j], z[j], al[j], be[j], *lin_states[j])
