@@ -319,6 +319,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
+    ap.add_argument("--only", choices=["c4", "c5"], default=None,
+                    help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path is measured on one GPU only (batch-1 decode attention on one "
@@ -326,6 +328,13 @@ def main():
         sys.exit(2)
     if a.calibrate_copy:
         calibrate_copy()
+        return
+
+    if a.only == "c4":
+        print(json.dumps({"c4_prefill_chunk_512": bench_prefill(a.steps, a.warmup, 0xC0FFEE + 4)}))
+        return
+    if a.only == "c5":
+        print(json.dumps({"c5_token_sweep_48_layers": bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)}))
         return
 
     Hq, Hkv, d, L = 32, 2, 256, 32768

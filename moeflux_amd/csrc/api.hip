@@ -265,6 +265,12 @@ static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
 // n_tok tokens whose K/V rows are already in the cache (the last n_tok positions).
 static int sdpa_dev(Ctx *c, FullLayer *f, int n_tok, const float *q, const float *gate, float *out) {
     if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
+    if (!c->forced_splits && !c->partial_only &&
+        sdpa_prefill_applies(c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads, n_tok, f->len,
+                             c->num_cus))
+        return launch_sdpa_prefill(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
+                                   c->cfg.head_dim, n_tok, f->len, c->plane_elems, f->k, f->v, q, gate, out,
+                                   c->num_cus);
     if (n_tok > 1) MFA_TRY(ensure_workspace(c, n_tok, f->len));
     return launch_sdpa(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
                        c->cfg.head_dim, n_tok, f->len, c->plane_elems, f->k, f->v, q, gate, out,

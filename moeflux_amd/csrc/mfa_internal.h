@@ -179,6 +179,12 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
                 int forced_splits, int partial_only = 0);
+// sdpa_prefill.hip: the same contract for a chunk whose rows fill the machine without
+// splitting the cache (no workspace, one launch).
+bool sdpa_prefill_applies(int kv_dtype, int Hq, int Hkv, int n_tok, int64_t kv_len, int num_cus);
+int launch_sdpa_prefill(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
+                        size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
+                        const float *gate, float *out, int num_cus);
 // Scatter `n_rows` row-major rows ([n_rows, Hkv*D], f32 or bf16 source) into the
 // tiled planes starting at position pos0.
 int launch_kv_scatter(hipStream_t stream, int kv_dtype, int src_is_bf16, int Hkv, int D,

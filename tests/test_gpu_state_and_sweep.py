@@ -40,6 +40,48 @@ def test_prefill_attn_equals_the_token_loop(mfa, oracle, T, L0):
     assert np.array_equal(ke, k) and np.array_equal(ve, v)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_prefill_attn_few_tokens_after_a_long_cache(mfa, oracle, bf16):
+    """A short chunk behind a long cache has too few rows to fill the machine, so the cache
+    is split over workgroups (the decode kernel on 16-row groups of (token, head)) and
+    merged; a ragged last row group (5 tokens x 4 heads = 20 rows) is part of the case."""
+    Hq, Hkv, d, T, L0 = 8, 2, 128, 5, 3000
+    rng = np.random.default_rng(31)
+    k = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    v = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    if bf16:
+        k, v = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k, v))
+    q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+    with _full_ctx(mfa, Hq, Hkv, d, 3072, bf16=bf16) as c:
+        c.kv_import(0, k[:L0], v[:L0])
+        out = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+    assert rel_err(out, ref) <= (1e-4 if bf16 else TOL_F32)
+
+
+@pytest.mark.parametrize("Hq,Hkv,d,T,L0,bf16", [(32, 2, 256, 70, 100, True), (8, 2, 64, 200, 0, False),
+                                                (32, 2, 256, 40, 9, False), (16, 4, 64, 130, 77, True),
+                                                (32, 4, 128, 1100, 50, True), (32, 16, 64, 2100, 0, True),
+                                                (32, 16, 64, 2050, 3, False)])
+def test_prefill_attn_shapes(mfa, oracle, Hq, Hkv, d, T, L0, bf16):
+    """The chunk kernel (one wave per 16-row group, K/V blocks staged in LDS) over head
+    dims, group sizes, ragged row counts and one or two row groups per wave."""
+    rng = np.random.default_rng(T + L0)
+    k = rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)
+    v = rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)
+    if bf16:
+        k, v = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k, v))
+    q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+    with _full_ctx(mfa, Hq, Hkv, d, L0 + T, bf16=bf16) as c:
+        if L0:
+            c.kv_import(0, k[:L0], v[:L0])
+        out = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+    assert rel_err(out, ref) <= (1e-4 if bf16 else TOL_F32)
+
+
 def test_prefill_attn_bf16_chunk_of_512(mfa, oracle):
     """BASELINE config 4, attention half: 512 tokens, 32 Q / 4 KV heads, d=128, bf16 values,
     from an empty cache."""
