@@ -8,8 +8,8 @@
 //
 //   gdn_chunk_pre_kernel    everything that does not depend on the state, for all T
 //                           tokens at once: conv + SiLU, per-head q/k norm, decay, beta.
-//   gdn_chunk_recur_kernel  one workgroup per value head keeps the state in registers
-//                           (8 lanes per row) across the whole chunk; the state is read
+//   gdn_chunk_recur_kernel  a workgroup keeps 16 rows of one value head's state in registers
+//                           (16 lanes per row) across the whole chunk; the state is read
 //                           once and written once per chunk instead of once per token.
 //                           k^, q^, v, g, beta of a slab of tokens are staged in LDS.
 //   gdn_chunk_post_kernel   gated RMS norm for all (token, head) pairs, and the conv
@@ -30,9 +30,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
     const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
     const float *__restrict__ ring, const float *__restrict__ qkv, const float *__restrict__ alpha,
     const float *__restrict__ beta, float *__restrict__ qn, float *__restrict__ kn,
-    float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg) {
+    float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg, float *__restrict__ kq) {
     static_assert(2 * DK <= 256, "one workgroup covers a k-head's q and k channels");
     __shared__ float s_part[4];
+    __shared__ float s_qk[2 * DK];
     const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x;
     const int C = 2 * Hk * DK + Hv * DV;
     const int nvb = (Hv * DV + 255) / 256;
@@ -58,6 +59,16 @@ __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
             v *= is_q ? inv_scale * inv_scale : inv_scale;
             if (is_q) qn[((size_t)t * Hk + y) * DK + tid] = v;
             else kn[((size_t)t * Hk + y) * DK + (tid - DK)] = v;
+            s_qk[tid] = v;
+        }
+        // k^ . q^ of the token, for the recurrence's read-out
+        __syncthreads();
+        if (tid < 64) {
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < DK / 64; i++) d = fmaf(s_qk[tid + 64 * i], s_qk[DK + tid + 64 * i], d);
+            d = group_sum<64>(d);
+            if (tid == 0) kq[(size_t)t * Hk + y] = d;
         }
     } else if (y < Hk + nvb) {
         const int i = (y - Hk) * 256 + tid;
@@ -73,55 +84,103 @@ __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
     }
 }
 
-// grid Hv, DV*8 threads.  o_raw [T, Hv*DV] receives the un-normalised read-outs.
+// grid (Hv, DV/16), 256 threads: a workgroup keeps 16 rows of one head's state in registers
+// across the chunk, 16 lanes per row (rows are independent, so a head's rows are spread
+// over DV/16 workgroups and every CU gets one).  o_raw [T, Hv*DV] receives the
+// un-normalised read-outs.
 template <int DK, int DV>
-__global__ __launch_bounds__(DV * 8) void gdn_chunk_recur_kernel(
+__global__ __launch_bounds__(256) void gdn_chunk_recur_kernel(
     int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ kn,
     const float *__restrict__ vv, const float *__restrict__ gd, const float *__restrict__ bg,
-    float *__restrict__ ssm, float *__restrict__ o_raw) {
-    constexpr int NI = DK / 32;
-    constexpr int NT = DV * 8;
+    const float *__restrict__ kq, float *__restrict__ ssm, float *__restrict__ o_raw) {
+    constexpr int NI = DK / 64;
+    constexpr int NT = 256, ROWS = 16;
     __shared__ __align__(16) float s_k[kSlab][DK];
     __shared__ __align__(16) float s_q[kSlab][DK];
-    __shared__ float s_v[kSlab][DV];
-    __shared__ float s_g[kSlab], s_b[kSlab];
+    __shared__ float s_v[kSlab][ROWS];
+    __shared__ float4 s_sc[kSlab];  // decay, beta gate, k . q
     const int tid = threadIdx.x, vh = blockIdx.x, kh = vh / (Hv / Hk);
-    const int r = tid >> 3, j = tid & 7;
-    float *srow = ssm + ((size_t)vh * DV + r) * DK + 4 * j;
+    const int row0 = blockIdx.y * ROWS;
+    const int r = tid >> 4, j = tid & 15;
+    float *srow = ssm + ((size_t)vh * DV + row0 + r) * DK + 4 * j;
     float4 s[NI];
 #pragma unroll
-    for (int i = 0; i < NI; i++) s[i] = *(const float4 *)(srow + 32 * i);
+    for (int i = 0; i < NI; i++) s[i] = *(const float4 *)(srow + 64 * i);
 
+    // A slab's operands travel global -> registers -> LDS; the registers are loaded one slab
+    // ahead, while the previous slab is being computed on.  Tokens past the end of the chunk
+    // re-read its last token (never used).
+    constexpr int KQ_T = kSlab * (DK / 4) / NT;  // float4 of k^ (and of q^) per thread
+    constexpr int V_T = kSlab * ROWS / NT;       // floats of v per thread
+    static_assert(kSlab * (DK / 4) % NT == 0 && kSlab * ROWS % NT == 0 && kSlab <= NT, "slab staging");
+    float4 pk[KQ_T], pq[KQ_T], psc;
+    float pv[V_T];
+    auto prefetch = [&](int t0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < KQ_T; u++) {
+            const int i = tid + u * NT;
+            int t = t0 + i / (DK / 4);
+            if (t > T - 1) t = T - 1;
+            const size_t src = ((size_t)t * Hk + kh) * DK + (i % (DK / 4)) * 4;
+            pk[u] = load_f4(kn + src);
+            pq[u] = load_f4(qn + src);
+        }
+#pragma unroll
+        for (int u = 0; u < V_T; u++) {
+            const int i = tid + u * NT;
+            int t = t0 + i / ROWS;
+            if (t > T - 1) t = T - 1;
+            pv[u] = vv[((size_t)t * Hv + vh) * DV + row0 + i % ROWS];
+        }
+        {
+            int t = t0 + (tid < kSlab ? tid : 0);
+            if (t > T - 1) t = T - 1;
+            psc = float4{gd[(size_t)t * Hv + vh], bg[(size_t)t * Hv + vh], kq[(size_t)t * Hk + kh], 0.f};
+        }
+    };
+    prefetch(0);
     for (int t0 = 0; t0 < T; t0 += kSlab) {
         const int nt = (T - t0 < kSlab) ? T - t0 : kSlab;
         __syncthreads();  // the previous slab has been consumed
-        for (int i = tid; i < nt * DK; i += NT) {
-            const int tt = i / DK, x = i % DK;
-            s_k[tt][x] = kn[((size_t)(t0 + tt) * Hk + kh) * DK + x];
-            s_q[tt][x] = qn[((size_t)(t0 + tt) * Hk + kh) * DK + x];
+#pragma unroll
+        for (int u = 0; u < KQ_T; u++) {
+            const int i = tid + u * NT;
+            *(float4 *)&s_k[i / (DK / 4)][(i % (DK / 4)) * 4] = pk[u];
+            *(float4 *)&s_q[i / (DK / 4)][(i % (DK / 4)) * 4] = pq[u];
         }
-        for (int i = tid; i < nt * DV; i += NT) {
-            const int tt = i / DV, x = i % DV;
-            s_v[tt][x] = vv[((size_t)(t0 + tt) * Hv + vh) * DV + x];
+#pragma unroll
+        for (int u = 0; u < V_T; u++) {
+            const int i = tid + u * NT;
+            s_v[i / ROWS][i % ROWS] = pv[u];
         }
-        if (tid < nt) {
-            s_g[tid] = gd[(size_t)(t0 + tid) * Hv + vh];
-            s_b[tid] = bg[(size_t)(t0 + tid) * Hv + vh];
-        }
+        if (tid < kSlab) s_sc[tid] = psc;
         __syncthreads();
-        for (int tt = 0; tt < nt; tt++) {
+        prefetch(t0 + kSlab);
+        // One instruction stream per SIMD: what counts is the instruction count per token.
+        // Groups of 4 tokens are written out so that their LDS reads go out together, with
+        // immediate offsets, and nothing is copied between registers.
+        auto token = [&](int tt) __attribute__((always_inline)) {
             float4 kk[NI], qq[NI];
 #pragma unroll
             for (int i = 0; i < NI; i++) {
-                kk[i] = *(const float4 *)(&s_k[tt][32 * i + 4 * j]);
-                qq[i] = *(const float4 *)(&s_q[tt][32 * i + 4 * j]);
+                kk[i] = *(const float4 *)(&s_k[tt][64 * i + 4 * j]);
+                qq[i] = *(const float4 *)(&s_q[tt][64 * i + 4 * j]);
             }
-            const float o = delta_row<DK>(s, kk, qq, s_g[tt], s_b[tt], s_v[tt][r]);
-            if (j == 0) o_raw[((size_t)(t0 + tt) * Hv + vh) * DV + r] = o;
+            const float4 sc = s_sc[tt];
+            const float o = delta_row16<DK>(s, kk, qq, sc.x, sc.y, s_v[tt][r], sc.z);
+            if (j == 0) o_raw[((size_t)(t0 + tt) * Hv + vh) * DV + row0 + r] = o;
+        };
+        int tt = 0;
+        for (; tt + 4 <= nt; tt += 4) {
+            token(tt);
+            token(tt + 1);
+            token(tt + 2);
+            token(tt + 3);
         }
+        for (; tt < nt; tt++) token(tt);
     }
 #pragma unroll
-    for (int i = 0; i < NI; i++) *(float4 *)(srow + 32 * i) = s[i];
+    for (int i = 0; i < NI; i++) *(float4 *)(srow + 64 * i) = s[i];
 }
 
 // grid (T, Hv) for the gated norm (shaders.metal:1337-1370) plus, at x == T, blocks that
@@ -154,7 +213,7 @@ __global__ __launch_bounds__(128) void gdn_chunk_post_kernel(
 }
 
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T) {
-    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 2 * (size_t)Hv);
+    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 2 * (size_t)Hv + (size_t)Hk);
 }
 
 int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
@@ -173,19 +232,20 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
     float *o_raw = vv + (size_t)T * Hv * dv;
     float *gd = o_raw + (size_t)T * Hv * dv;
     float *bg = gd + (size_t)T * Hv;
+    float *kq = bg + (size_t)T * Hv;
     const int nvb = (Hv * dv + 255) / 256;
     if (dk == 128) {
         hipLaunchKernelGGL((gdn_chunk_pre_kernel<128>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
                            K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
-                           vv, gd, bg);
-        hipLaunchKernelGGL((gdn_chunk_recur_kernel<128, 128>), dim3(Hv), dim3(1024), 0, s, Hk, Hv, T, qn,
-                           kn, vv, gd, bg, ssm, o_raw);
+                           vv, gd, bg, kq);
+        hipLaunchKernelGGL((gdn_chunk_recur_kernel<128, 128>), dim3(Hv, 128 / 16), dim3(256), 0, s, Hk, Hv, T, qn,
+                           kn, vv, gd, bg, kq, ssm, o_raw);
     } else {
         hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
                            K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
-                           vv, gd, bg);
-        hipLaunchKernelGGL((gdn_chunk_recur_kernel<64, 64>), dim3(Hv), dim3(512), 0, s, Hk, Hv, T, qn, kn,
-                           vv, gd, bg, ssm, o_raw);
+                           vv, gd, bg, kq);
+        hipLaunchKernelGGL((gdn_chunk_recur_kernel<64, 64>), dim3(Hv, 64 / 16), dim3(256), 0, s, Hk, Hv, T, qn, kn,
+                           vv, gd, bg, kq, ssm, o_raw);
     }
     MFA_HIP(hipGetLastError());
     hipLaunchKernelGGL(gdn_chunk_post_kernel, dim3(T + 1, Hv), dim3(128), 0, s, Hv, dv, T, C, K, step, eps,

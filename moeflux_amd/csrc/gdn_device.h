@@ -5,6 +5,14 @@
 
 namespace mfa {
 
+// A 16-byte load as a register value (assigning through a float4 pointer is a struct copy,
+// which the compiler may leave as a memcpy into a stack slot when the target is an array).
+typedef float gdn_f32x4 __attribute__((ext_vector_type(4)));
+__device__ inline float4 load_f4(const float *p) {
+    const gdn_f32x4 v = *reinterpret_cast<const gdn_f32x4 *>(p);
+    return float4{v.x, v.y, v.z, v.w};
+}
+
 __device__ inline float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
 // v + (v of the lane selected by a DPP control word); no LDS round trip.
@@ -64,6 +72,41 @@ __device__ inline float delta_row(float4 (&s)[DK / 32], const float4 (&kk)[DK / 
         o = fmaf(s[i].w, qq[i].w, o);
     }
     return group_sum<8>(o);
+}
+
+// The same update for a wave that walks a whole chunk, with a row spread over 16 lanes
+// (lane j owns floats 64*i + 4*j .. +3 for i < DK/64) and the dependent chain per token
+// kept short: both dot products are taken on the row before this token's update,
+//   kv = g (S k),  delta = beta (v - kv),  out = g (S q) + delta (k . q),  S <- g S + delta k^T,
+// which equals decay / kv_mem / delta / rank-1 update / read-out of the updated row
+// (crates/moeflux/src/riir/linear_attn.rs:383-410) up to rounding.  kq = k . q of the token.
+template <int DK>
+__device__ inline float delta_row16(float4 (&s)[DK / 64], const float4 (&kk)[DK / 64],
+                                    const float4 (&qq)[DK / 64], float g, float beta, float v, float kq) {
+    constexpr int NI = DK / 64;
+    float a0 = 0.f, a1 = 0.f, c0 = 0.f, c1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        a0 = fmaf(s[i].x, kk[i].x, a0);
+        a1 = fmaf(s[i].y, kk[i].y, a1);
+        c0 = fmaf(s[i].x, qq[i].x, c0);
+        c1 = fmaf(s[i].y, qq[i].y, c1);
+        a0 = fmaf(s[i].z, kk[i].z, a0);
+        a1 = fmaf(s[i].w, kk[i].w, a1);
+        c0 = fmaf(s[i].z, qq[i].z, c0);
+        c1 = fmaf(s[i].w, qq[i].w, c1);
+    }
+    const float sk = group_sum<16>(a0 + a1);
+    const float sq = group_sum<16>(c0 + c1);
+    const float delta = (v - g * sk) * beta;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        s[i].x = fmaf(kk[i].x, delta, g * s[i].x);
+        s[i].y = fmaf(kk[i].y, delta, g * s[i].y);
+        s[i].z = fmaf(kk[i].z, delta, g * s[i].z);
+        s[i].w = fmaf(kk[i].w, delta, g * s[i].w);
+    }
+    return fmaf(delta, kq, g * sq);
 }
 
 // Depthwise conv + SiLU of channel ch for the input numbered `step + t` of the layer

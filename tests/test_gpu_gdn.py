@@ -97,10 +97,12 @@ def test_gdn_kernel_hooks(mfa, oracle):
 
 
 @pytest.mark.parametrize("T", [2, 3, 4, 5, 37, 100])
-def test_chunk_equals_token_loop_bit_for_bit(mfa, T):
-    """The chunk kernels do, token for token, the arithmetic of the single-step kernel
-    (riir/mod.rs:1196-1214: a prompt is a loop of steps); T below, at and above the conv
-    width exercises the history ring on both sides of the chunk boundary."""
+def test_chunk_equals_token_loop(mfa, T):
+    """The chunk kernels do, token for token, the operations of the single-step kernel
+    (riir/mod.rs:1196-1214: a prompt is a loop of steps) and differ from it only in how a
+    state row's dot products are grouped over lanes (16 lanes per row against 8); the conv
+    history is copied and must be identical.  T below, at and above the conv width
+    exercises the history ring on both sides of the chunk boundary."""
     case = GdnCase(40 + T, 4, 8, 128, 128, T=T)
     with _ctx(mfa, case, num_layers=2) as c:
         for layer in (0, 1):
@@ -113,9 +115,9 @@ def test_chunk_equals_token_loop_bit_for_bit(mfa, T):
         extra = GdnCase(99, 4, 8, 128, 128, T=1)
         n0 = c.gdn_step(0, extra.qkv[0], extra.z[0], extra.alpha[0], extra.beta[0])
         n1 = c.gdn_step(1, extra.qkv[0], extra.z[0], extra.alpha[0], extra.beta[0])
-    assert np.array_equal(chunk, loop)
-    assert np.array_equal(s0[0], s1[0]) and np.array_equal(s0[1], s1[1])
-    assert np.array_equal(n0, n1)
+    assert rel_err(chunk, loop) <= 2e-6
+    assert np.array_equal(s0[0], s1[0]) and rel_err(s0[1], s1[1]) <= 2e-6
+    assert rel_err(n0, n1) <= 2e-6
     ref_out, ref_conv, ref_ssm = case.oracle()
     assert rel_err(chunk, ref_out) <= TOL_F32
     assert np.array_equal(s0[0].reshape(-1), ref_conv) and rel_err(s0[1], ref_ssm) <= TOL_F32
