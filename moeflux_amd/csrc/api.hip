@@ -547,8 +547,11 @@ int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv
     if (T == 1) return gdn_step_dev(c, l, qkv_in_dev, z_dev, alpha_dev, beta_dev, out_dev);
     if (!l->w.set) return fail(MFA_ERR_INVALID, "linear layer weights not set (mfa_set_linear_weights)");
     const mfa_config &g = c->cfg;
+    // Long prompts go through in segments, which bounds the scratch (about 57 KB per token
+    // at the 16/32-head, 128-wide shape); the ring and the state carry over as between calls.
+    const int kSeg = 4096;
     const size_t need = gdn_chunk_scratch_elems(g.linear_num_k_heads, g.linear_num_v_heads,
-                                                g.linear_key_dim, g.linear_value_dim, T);
+                                                g.linear_key_dim, g.linear_value_dim, T < kSeg ? T : kSeg);
     if (need > c->gdn_scratch_elems) {
         MFA_HIP(hipStreamSynchronize(c->stream));
         if (c->gdn_scratch) MFA_HIP(hipFree(c->gdn_scratch));
@@ -557,11 +560,15 @@ int mfa_prefill_gdn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *qkv
         MFA_HIP(hipMalloc((void **)&c->gdn_scratch, need * sizeof(float)));
         c->gdn_scratch_elems = need;
     }
-    MFA_TRY(launch_gdn_chunk(c->stream, g.linear_num_k_heads, g.linear_num_v_heads, g.linear_key_dim,
-                             g.linear_value_dim, g.conv_kernel_size, g.rms_norm_eps, T, l->w,
-                             l->conv_ring, l->step, l->ssm, qkv_in_dev, z_dev, alpha_dev, beta_dev,
-                             c->gdn_scratch, out_dev));
-    l->step += T;
+    const size_t C = (size_t)c->conv_dim(), tv = (size_t)c->v_total(), Hv = (size_t)g.linear_num_v_heads;
+    for (int off = 0; off < T; off += kSeg) {
+        const int n = T - off < kSeg ? T - off : kSeg;
+        MFA_TRY(launch_gdn_chunk(c->stream, g.linear_num_k_heads, g.linear_num_v_heads, g.linear_key_dim,
+                                 g.linear_value_dim, g.conv_kernel_size, g.rms_norm_eps, n, l->w,
+                                 l->conv_ring, l->step, l->ssm, qkv_in_dev + off * C, z_dev + off * tv,
+                                 alpha_dev + off * Hv, beta_dev + off * Hv, c->gdn_scratch, out_dev + off * tv));
+        l->step += n;
+    }
     return MFA_OK;
 }
 

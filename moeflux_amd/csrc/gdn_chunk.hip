@@ -30,7 +30,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
     const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
     const float *__restrict__ ring, const float *__restrict__ qkv, const float *__restrict__ alpha,
     const float *__restrict__ beta, float *__restrict__ qn, float *__restrict__ kn,
-    float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg, float *__restrict__ kq) {
+    float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg, float *__restrict__ kq,
+    float *__restrict__ lg) {
     static_assert(2 * DK <= 256, "one workgroup covers a k-head's q and k channels");
     __shared__ float s_part[4];
     __shared__ float s_qk[2 * DK];
@@ -79,6 +80,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
             const float a_cap = expf(a_log[h]);
             const float sp = logf(1.0f + expf(alpha[(size_t)t * Hv + h] + bf16_bits_to_f32(dt_bias[h])));
             gd[(size_t)t * Hv + h] = expf(-a_cap * sp);
+            lg[(size_t)t * Hv + h] = -a_cap * sp;  // log of the decay, for the blocked form
             bg[(size_t)t * Hv + h] = 1.0f / (1.0f + expf(-beta[(size_t)t * Hv + h]));
         }
     }
@@ -212,8 +214,16 @@ __global__ __launch_bounds__(128) void gdn_chunk_post_kernel(
         out[base + i] = o_raw[base + i] * inv * bf16_bits_to_f32(norm_w[i]) * silu_f(z[base + i]);
 }
 
+// Chunks of at least this many tokens take the blocked form on the matrix cores; shorter
+// ones step the recurrence token by token.
+static constexpr int kWyMinTokens = 48;
+
+static size_t chunk_common_elems(int Hk, int Hv, int dk, int dv, int T) {
+    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 3 * (size_t)Hv + (size_t)Hk);
+}
+
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T) {
-    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 2 * (size_t)Hv + (size_t)Hk);
+    return chunk_common_elems(Hk, Hv, dk, dv, T) + (T >= kWyMinTokens ? gdn_wy_scratch_elems(Hv, dk, dv, T) : 0);
 }
 
 int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
@@ -232,18 +242,26 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
     float *o_raw = vv + (size_t)T * Hv * dv;
     float *gd = o_raw + (size_t)T * Hv * dv;
     float *bg = gd + (size_t)T * Hv;
-    float *kq = bg + (size_t)T * Hv;
+    float *lg = bg + (size_t)T * Hv;
+    float *kq = lg + (size_t)T * Hv;
+    float *wy = scratch + chunk_common_elems(Hk, Hv, dk, dv, T);
     const int nvb = (Hv * dv + 255) / 256;
-    if (dk == 128) {
+    const bool blocked = T >= kWyMinTokens;
+    if (dk == 128)
         hipLaunchKernelGGL((gdn_chunk_pre_kernel<128>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
                            K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
-                           vv, gd, bg, kq);
+                           vv, gd, bg, kq, lg);
+    else
+        hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
+                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
+                           vv, gd, bg, kq, lg);
+    MFA_HIP(hipGetLastError());
+    if (blocked) {
+        MFA_TRY(launch_gdn_wy(s, Hk, Hv, dk, dv, T, qn, kn, vv, lg, bg, wy, ssm, o_raw));
+    } else if (dk == 128) {
         hipLaunchKernelGGL((gdn_chunk_recur_kernel<128, 128>), dim3(Hv, 128 / 16), dim3(256), 0, s, Hk, Hv, T, qn,
                            kn, vv, gd, bg, kq, ssm, o_raw);
     } else {
-        hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
-                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
-                           vv, gd, bg, kq);
         hipLaunchKernelGGL((gdn_chunk_recur_kernel<64, 64>), dim3(Hv, 64 / 16), dim3(256), 0, s, Hk, Hv, T, qn, kn,
                            vv, gd, bg, kq, ssm, o_raw);
     }

@@ -217,6 +217,12 @@ int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float 
 // gdn_chunk.hip: T tokens through one layer (three launches); scratch holds
 // gdn_chunk_scratch_elems floats.
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T);
+// gdn_wy.hip: the recurrence of a chunk in blocked form (blocks of 64 tokens) on the matrix
+// cores, from the per-token operands the chunk's first kernel prepares.
+size_t gdn_wy_scratch_elems(int Hv, int dk, int dv, int T);
+int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const float *qn, const float *kn,
+                  const float *vv, const float *lg, const float *bg, float *scratch, float *ssm,
+                  float *o_raw);
 int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
                      const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                      const float *qkv_in, const float *z, const float *alpha, const float *beta,
