@@ -21,6 +21,8 @@
 // 4 instructions i = 0..3 in which lane group g contributes value number 4g+i: then one
 // float4 (values 4g..4g+3) feeds the four instructions, and a D tile can be used as the
 // B operand of a contraction over its rows without moving data between lanes.
+#include <type_traits>
+
 #include "gdn_device.h"
 
 namespace mfa {
@@ -36,25 +38,47 @@ __device__ inline wy_f32x4 mfma4(float4 a, float4 b, wy_f32x4 acc) {
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
     return acc;
 }
+// The same four instructions on four accumulators: a dependent v_mfma has to wait for the
+// previous one to leave the pipeline, about three times its issue time, so long
+// contractions keep four independent chains going and add them at the end.
+struct Acc4 {
+    wy_f32x4 a[4];
+    __device__ Acc4() { a[0] = a[1] = a[2] = a[3] = wy_f32x4{0.f, 0.f, 0.f, 0.f}; }
+    __device__ wy_f32x4 sum() const { return (a[0] + a[1]) + (a[2] + a[3]); }
+};
+__device__ inline void mfma4x(float4 a, float4 b, Acc4 &acc) {
+    acc.a[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc.a[0], 0, 0, 0);
+    acc.a[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc.a[1], 0, 0, 0);
+    acc.a[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc.a[2], 0, 0, 0);
+    acc.a[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc.a[3], 0, 0, 0);
+}
 __device__ inline float4 lds_f4(const float *p) {
     const gdn_f32x4 v = *reinterpret_cast<const gdn_f32x4 *>(p);
     return float4{v.x, v.y, v.z, v.w};
 }
 __device__ inline float4 as_f4(wy_f32x4 v) { return float4{v[0], v[1], v[2], v[3]}; }
+// a 16-byte load kept as a vector register value (members of a struct of operands)
+__device__ inline wy_f32x4 load_v4(const float *p) { return *reinterpret_cast<const wy_f32x4 *>(p); }
 
-// Per (block, value head) outputs, block-major then head:
-//   Wc [64][DK], Uc [64][DV], Mc [64][64], KdT [DK][64] (= diag(e^{L_C-L}) K, transposed),
+// Per (block, value head) outputs, block-major then head, each cut into 16x16 tiles that
+// are stored the way the recurrence kernel's lanes read them, 16 bytes per lane and
+// 1 KiB per tile (a row-major matrix read as an A operand has neighbouring lanes 512
+// bytes apart, which the memory pipeline serves at a fraction of its rate):
+//   Wt [token tile w][col tile c], Qt likewise, Mt [w][token tile tau], Kt [col tile c][tau]
+//   (= diag(e^{L_C-L}) K transposed): lane (m, g) holds X[16 row-tile + m][16 col-tile + 4g + i];
+//   Ut [w][col tile c]: lane (n, g) holds U[16w + 4g + i][16c + n]  (a D tile as computed);
 //   eL [64] (e^{L_t}; eL[63] = e^{L_C} because padded tokens do not decay).
 // Tokens past the end of the chunk are padded with beta = 0, log g = 0, k = q = v = 0.
 //
-// grid (blocks, Hv), 256 threads.
+// grid (Hv, blocks), 256 threads.
 template <int DK>
 __global__ __launch_bounds__(256) void gdn_wy_kernel(
     int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ kn,
     const float *__restrict__ vv, const float *__restrict__ lg, const float *__restrict__ bg,
-    float *__restrict__ Wc, float *__restrict__ Uc, float *__restrict__ Mc, float *__restrict__ KdT,
-    float *__restrict__ eLc) {
+    float *__restrict__ Wt, float *__restrict__ Qt, float *__restrict__ Ut, float *__restrict__ Mt,
+    float *__restrict__ Kt, float *__restrict__ eLc) {
     constexpr int DV = DK;
+    constexpr int NK = DK / 16;
     constexpr int LDK = DK + 4;  // row strides chosen so that 16-byte row reads by 8 lanes hit all banks
     constexpr int LDC = kC + 4;
     constexpr int NCT = DK / 64;  // 16-wide column tiles of W (and of U) per wave
@@ -64,7 +88,9 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     __shared__ __align__(16) float sT[kC][LDC];
     __shared__ __align__(16) float sL[kC], sB[kC], sCw[kC];
 
-    const int blk = blockIdx.x, vh = blockIdx.y, kh = vh / (Hv / Hk);
+    // heads along x: a head's blocks are produced on the XCD whose L2 the recurrence kernel
+    // (heads along x as well) will read them through
+    const int vh = blockIdx.x, blk = blockIdx.y, kh = vh / (Hv / Hk);
     const int t0 = blk * kC;
     const int nt = (T - t0 < kC) ? T - t0 : kC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -106,10 +132,11 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
         const int I = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
         const int J = idx - I * (I + 1) / 2;
         const float(*X)[LDK] = kind ? sQ : sK;
-        wy_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        Acc4 acc4;
 #pragma unroll
         for (int s = 0; s < DK / 16; s++)
-            acc = mfma4(lds_f4(&X[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc);
+            mfma4x(lds_f4(&X[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc4);
+        const wy_f32x4 acc = acc4.sum();
         // lane (n = m, g) holds rows 16I + 4g + i of column 16J + n
         const int col = 16 * J + m;
 #pragma unroll
@@ -118,48 +145,80 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
             const float dl = sL[row] - sL[col];
             const float d = expf(dl < 0.f ? dl : 0.f);
             if (kind == 0) sA[row][col] = (col < row) ? sB[row] * d * acc[i] : 0.f;
-            else Mc[slot * kC * kC + (size_t)row * kC + col] = (col <= row) ? d * acc[i] : 0.f;
+            else  // to tile (I, J) in A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
+                Mt[((slot * 4 + I) * 4 + J) * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = (col <= row) ? d * acc[i] : 0.f;
         }
+    }
+    for (int i = tid; i < 4 * NK * 64; i += 256) {  // q^ tiles, before v takes its place
+        const int tile = i >> 6, l = i & 63, w = tile / NK, c = tile % NK;
+        *(float4 *)(Qt + (slot * 4 * NK + tile) * 256 + l * 4) = lds_f4(&sQ[16 * w + (l & 15)][16 * c + 4 * (l >> 4)]);
     }
     __syncthreads();
 
-    // ---- phase 2: T = (I + A)^-1 by forward substitution, one column per lane of wave 0;
-    //      the other waves write diag(e^{L_C - L}) K transposed and bring in v --------------
-    if (wave == 0) {
-        float t[kC];
-#pragma unroll
-        for (int i = 0; i < kC; i++) {
-            float acc = (i == lane) ? 1.f : 0.f;
-#pragma unroll
-            for (int j4 = 0; j4 < i; j4 += 4) {
-                const float4 a = lds_f4(&sA[i][j4]);  // the same address in every lane
-                acc = fmaf(-a.x, t[j4], acc);
-                if (j4 + 1 < i) acc = fmaf(-a.y, t[j4 + 1], acc);
-                if (j4 + 2 < i) acc = fmaf(-a.z, t[j4 + 2], acc);
-                if (j4 + 3 < i) acc = fmaf(-a.w, t[j4 + 3], acc);
-            }
-            t[i] = acc;
-            sT[i][lane] = acc;
-        }
-    } else {
+    // ---- phase 2: diag(e^{L_C - L}) K transposed goes out, v comes in, and
+    //      T = (I + A)^-1 by blocks of 16: the diagonal blocks by forward substitution (one
+    //      per wave, a column per lane), the blocks below them level by level from
+    //      T_IJ = -T_II sum_{J <= K < I} A_IK T_KJ on the matrix cores -----------------------
+    {
         const float lc = sL[kC - 1];
-        for (int i = tid - 64; i < DK * (kC / 4); i += 192) {
-            const int kk = i % DK, j4 = (i / DK) * 4;
+        for (int i = tid; i < NK * 4 * 64; i += 256) {
+            const int tile = i >> 6, l = i & 63, c = tile >> 2, tau = tile & 3;
+            const int kk = 16 * c + (l & 15), j4 = 16 * tau + 4 * (l >> 4);
             float4 o;
             o.x = expf(lc - sL[j4 + 0]) * sK[j4 + 0][kk];
             o.y = expf(lc - sL[j4 + 1]) * sK[j4 + 1][kk];
             o.z = expf(lc - sL[j4 + 2]) * sK[j4 + 2][kk];
             o.w = expf(lc - sL[j4 + 3]) * sK[j4 + 3][kk];
-            *(float4 *)(KdT + slot * DK * kC + (size_t)kk * kC + j4) = o;
+            *(float4 *)(Kt + (slot * NK * 4 + tile) * 256 + l * 4) = o;
         }
-        for (int i = tid - 64; i < kC * (DV / 4); i += 192) {
+        for (int i = tid; i < kC * (DV / 4); i += 256) {
             const int tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
             float4 a = {0.f, 0.f, 0.f, 0.f};
             if (tt < nt) a = load_f4(vv + ((size_t)(t0 + tt) * Hv + vh) * DV + x);
             *(float4 *)&sQ[tt][x] = a;
         }
     }
+    {
+        // block `wave`; the four lane groups compute the same 16 columns, group 0 stores
+        const int r0 = 16 * wave;
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float acc = (i == m) ? 1.f : 0.f;
+#pragma unroll
+            for (int j4 = 0; j4 < i; j4 += 4) {
+                const float4 a = lds_f4(&sA[r0 + i][r0 + j4]);  // the same address in every lane
+                acc = fmaf(-a.x, t[j4], acc);
+                if (j4 + 1 < i) acc = fmaf(-a.y, t[j4 + 1], acc);
+                if (j4 + 2 < i) acc = fmaf(-a.z, t[j4 + 2], acc);
+                if (j4 + 3 < i) acc = fmaf(-a.w, t[j4 + 3], acc);
+            }
+            t[i] = acc;
+            if (g == 0) sT[r0 + i][r0 + m] = acc;
+        }
+    }
     __syncthreads();
+#pragma unroll
+    for (int lvl = 1; lvl < 4; lvl++) {
+        if (wave < 4 - lvl) {  // block (I, J) = (wave + lvl, wave)
+            const int I = wave + lvl, J = wave;
+            wy_f32x4 x = {0.f, 0.f, 0.f, 0.f};
+            for (int K = J; K < I; K++) {
+                float4 bt;
+                bt.x = sT[16 * K + 4 * g + 0][16 * J + m];
+                bt.y = sT[16 * K + 4 * g + 1][16 * J + m];
+                bt.z = sT[16 * K + 4 * g + 2][16 * J + m];
+                bt.w = sT[16 * K + 4 * g + 3][16 * J + m];
+                x = mfma4(lds_f4(&sA[16 * I + m][16 * K + 4 * g]), bt, x);
+            }
+            // x is held as rows 4g+i of column m: already the B operand of T_II x
+            wy_f32x4 r = {0.f, 0.f, 0.f, 0.f};
+            r = mfma4(lds_f4(&sT[16 * I + m][16 * I + 4 * g]), as_f4(x), r);
+#pragma unroll
+            for (int i = 0; i < 4; i++) sT[16 * I + 4 * g + i][16 * J + m] = -r[i];
+        }
+        __syncthreads();
+    }
 
     // ---- phase 3: W = T diag(beta e^L) K and U = T diag(beta) V -------------------------
     // Wave w owns column tiles NCT*w .. of both; the K and V operands of those columns are
@@ -176,9 +235,7 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
             }
 #pragma unroll
     for (int tau = 0; tau < 4; tau++) {
-        wy_f32x4 aw[NCT], au[NCT];
-#pragma unroll
-        for (int ct = 0; ct < NCT; ct++) aw[ct] = au[ct] = wy_f32x4{0.f, 0.f, 0.f, 0.f};
+        Acc4 aw4[NCT], au4[NCT];
 #pragma unroll
         for (int s = 0; s <= tau; s++) {
             const float4 t4 = lds_f4(&sT[16 * tau + m][16 * s + 4 * g]);
@@ -187,18 +244,19 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
             const float4 tu = {t4.x * cb.x, t4.y * cb.y, t4.z * cb.z, t4.w * cb.w};
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) {
-                aw[ct] = mfma4(tw, float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, aw[ct]);
-                au[ct] = mfma4(tu, float4{bV[s][ct][0], bV[s][ct][1], bV[s][ct][2], bV[s][ct][3]}, au[ct]);
+                mfma4x(tw, float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, aw4[ct]);
+                mfma4x(tu, float4{bV[s][ct][0], bV[s][ct][1], bV[s][ct][2], bV[s][ct][3]}, au4[ct]);
             }
         }
 #pragma unroll
-        for (int ct = 0; ct < NCT; ct++)
+        for (int ct = 0; ct < NCT; ct++) {
+            const wy_f32x4 aw = aw4[ct].sum(), au = au4[ct].sum();
+            const size_t tile = (slot * 4 + tau) * NK + NCT * wave + ct;
+            // U as computed; W to A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
+            *reinterpret_cast<wy_f32x4 *>(Ut + tile * 256 + lane * 4) = au;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const size_t row = 16 * tau + 4 * g + i, col = 16 * (NCT * wave + ct) + m;
-                Wc[slot * kC * DK + row * DK + col] = aw[ct][i];
-                Uc[slot * kC * DV + row * DV + col] = au[ct][i];
-            }
+            for (int i = 0; i < 4; i++) Wt[tile * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = aw[i];
+        }
     }
 }
 
@@ -208,8 +266,8 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
 // block and the column tiles (DK/64)*w .. of the state update.
 template <int DK>
 __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
-    int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ Wc,
-    const float *__restrict__ Uc, const float *__restrict__ Mc, const float *__restrict__ KdT,
+    int Hk, int Hv, int T, const float *__restrict__ Wt, const float *__restrict__ Qt,
+    const float *__restrict__ Ut, const float *__restrict__ Mt, const float *__restrict__ Kt,
     const float *__restrict__ eLc, float *__restrict__ ssm, float *__restrict__ o_raw) {
     constexpr int DV = DK;
     constexpr int NK = DK / 16;   // column tiles of the state
@@ -217,7 +275,7 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
     __shared__ wy_f32x4 s_d[4][64];    // D tiles of the block, by token tile
     __shared__ wy_f32x4 s_st[NK][64];  // the updated state
 
-    const int vh = blockIdx.x, kh = vh / (Hv / Hk), row0 = blockIdx.y * 16;
+    const int vh = blockIdx.x, row0 = blockIdx.y * 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = lane & 15, g = lane >> 4;
     float *srow = ssm + ((size_t)vh * DV + row0 + m) * DK + 4 * g;
@@ -228,62 +286,99 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
         st[c] = wy_f32x4{v.x, v.y, v.z, v.w};
     }
 
+    // A block's operands live in registers and are requested one block ahead, all of them
+    // before the block's first barrier: the W and q^ rows of this wave's tokens and its U
+    // entries into the registers the block has just consumed, its M rows, e^L and the K
+    // columns of its share of the update into a second set (two blocks per loop pass,
+    // the sets swapping roles).  Requests past the last block re-read it.
     const int nblk = (T + kC - 1) / kC;
-    for (int blk = 0; blk < nblk; blk++) {
-        const int t0 = blk * kC;
-        const size_t slot = (size_t)blk * Hv + vh;
-        const float *Wb = Wc + slot * kC * DK, *Ub = Uc + slot * kC * DV, *Mb = Mc + slot * kC * kC;
-        const float *Kb = KdT + slot * DK * kC, *eL = eLc + slot * kC;
-        // ---- W S0^T and Q S0^T for this wave's 16 tokens ------------------------------
-        const int tq = t0 + 16 * wave + m;  // the token whose q^ row this lane supplies
-        const float *qrow = qn + ((size_t)(tq < T ? tq : T - 1) * Hk + kh) * DK + 4 * g;
-        const float *wrow = Wb + (size_t)(16 * wave + m) * DK + 4 * g;
-        wy_f32x4 p1 = {0.f, 0.f, 0.f, 0.f}, p2 = p1;
+    struct Late {
+        wy_f32x4 mt[4], kd[NKW][4], el;
+        float elc;
+    };
+    float4 pw[NK], pq[NK], pu;
+    auto slot_of = [&](int blk) { return (size_t)(blk < nblk ? blk : nblk - 1) * Hv + vh; };
+    auto fetch_wq = [&](int blk) __attribute__((always_inline)) {
+        const size_t off = (slot_of(blk) * 4 + wave) * NK * 256 + lane * 4;
 #pragma unroll
         for (int c = 0; c < NK; c++) {
-            const float4 aw = load_f4(wrow + 16 * c);
-            float4 aq = load_f4(qrow + 16 * c);
-            if (tq >= T) aq = float4{0.f, 0.f, 0.f, 0.f};
-            p1 = mfma4(aw, as_f4(st[c]), p1);
-            p2 = mfma4(aq, as_f4(st[c]), p2);
+            pw[c] = load_f4(Wt + off + c * 256);
+            pq[c] = load_f4(Qt + off + c * 256);
         }
+    };
+    auto fetch_u = [&](int blk) __attribute__((always_inline)) {
+        pu = load_f4(Ut + ((slot_of(blk) * 4 + wave) * NK + blockIdx.y) * 256 + lane * 4);
+    };
+    auto fetch_late = [&](Late &p, int blk) __attribute__((always_inline)) {
+        const size_t slot = slot_of(blk);
+#pragma unroll
+        for (int tau = 0; tau < 4; tau++)
+            p.mt[tau] = load_v4(Mt + ((slot * 4 + wave) * 4 + (tau <= wave ? tau : wave)) * 256 + lane * 4);
+        p.el = load_v4(eLc + slot * kC + 16 * wave + 4 * g);
+#pragma unroll
+        for (int kt = 0; kt < NKW; kt++)
+#pragma unroll
+            for (int tau = 0; tau < 4; tau++)
+                p.kd[kt][tau] = load_v4(Kt + ((slot * NK + NKW * wave + kt) * 4 + tau) * 256 + lane * 4);
+        p.elc = eLc[slot * kC + kC - 1];
+    };
+    auto block = [&](int blk, const Late &cur, Late &nxt) __attribute__((always_inline)) {
+        const int t0 = blk * kC;
+        // ---- W S0^T and Q S0^T for this wave's 16 tokens ------------------------------
+        Acc4 p1x, p2x;
+#pragma unroll
+        for (int c = 0; c < NK; c++) {
+            mfma4x(pw[c], as_f4(st[c]), p1x);
+            mfma4x(pq[c], as_f4(st[c]), p2x);
+        }
+        const wy_f32x4 p1 = p1x.sum(), p2 = p2x.sum();
+        fetch_wq(blk + 1);
         // ---- D = U - W S0^T: lane (n, g) holds tokens 16w+4g+i of state row row0+n ----
         wy_f32x4 d;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            d[i] = Ub[(size_t)(16 * wave + 4 * g + i) * DV + row0 + m] - p1[i];
+        d[0] = pu.x - p1[0]; d[1] = pu.y - p1[1]; d[2] = pu.z - p1[2]; d[3] = pu.w - p1[3];
+        fetch_u(blk + 1);
+        fetch_late(nxt, blk + 1);
         s_d[wave][lane] = d;
         __syncthreads();
         // ---- O = diag(e^L) Q S0^T + M D ------------------------------------------------
-        const float4 el = load_f4(eL + 16 * wave + 4 * g);
-        wy_f32x4 o = {el.x * p2[0], el.y * p2[1], el.z * p2[2], el.w * p2[3]};
-        for (int tau = 0; tau <= wave; tau++)
-            o = mfma4(load_f4(Mb + (size_t)(16 * wave + m) * kC + 16 * tau + 4 * g), as_f4(s_d[tau][lane]), o);
+        Acc4 ox;
+#pragma unroll
+        for (int tau = 0; tau < 4; tau++)
+            if (tau <= wave) mfma4x(as_f4(cur.mt[tau]), as_f4(s_d[tau][lane]), ox);
+        const wy_f32x4 o = cur.el * p2 + ox.sum();
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int t = t0 + 16 * wave + 4 * g + i;
             if (t < T) o_raw[((size_t)t * Hv + vh) * DV + row0 + m] = o[i];
         }
         // ---- S' = e^{L_C} S0 + D^T diag(e^{L_C-L}) K, column tiles NKW*w .. ------------
-        const float elc = eL[kC - 1];
+        // (written out per wave so that the state tile is a compile-time register choice)
+        auto update = [&](auto wtag) __attribute__((always_inline)) {
+            constexpr int w = decltype(wtag)::value;
 #pragma unroll
-        for (int kt = 0; kt < NKW; kt++) {
-            const int c = NKW * wave + kt;
-            wy_f32x4 acc;
-            // st[c] with a runtime c: pick it without indexing the register array
-            wy_f32x4 cur = st[0];
+            for (int kt = 0; kt < NKW; kt++) {
+                constexpr int c0 = NKW * w;
+                Acc4 ux;
 #pragma unroll
-            for (int cc = 1; cc < NK; cc++)
-                if (cc == c) cur = st[cc];
-            acc = wy_f32x4{elc * cur[0], elc * cur[1], elc * cur[2], elc * cur[3]};
-#pragma unroll
-            for (int tau = 0; tau < 4; tau++)
-                acc = mfma4(load_f4(Kb + (size_t)(16 * c + m) * kC + 16 * tau + 4 * g), as_f4(s_d[tau][lane]), acc);
-            s_st[c][lane] = acc;
-        }
+                for (int tau = 0; tau < 4; tau++) mfma4x(as_f4(cur.kd[kt][tau]), as_f4(s_d[tau][lane]), ux);
+                s_st[c0 + kt][lane] = st[c0 + kt] * cur.elc + ux.sum();
+            }
+        };
+        if (wave == 0) update(std::integral_constant<int, 0>{});
+        else if (wave == 1) update(std::integral_constant<int, 1>{});
+        else if (wave == 2) update(std::integral_constant<int, 2>{});
+        else update(std::integral_constant<int, 3>{});
         __syncthreads();
 #pragma unroll
         for (int c = 0; c < NK; c++) st[c] = s_st[c][lane];
+    };
+    Late la, lb;
+    fetch_wq(0);
+    fetch_u(0);
+    fetch_late(la, 0);
+    for (int blk = 0; blk < nblk; blk += 2) {
+        block(blk, la, lb);
+        if (blk + 1 < nblk) block(blk + 1, lb, la);  // uniform over the workgroup
     }
     if (wave == 0) {
 #pragma unroll
@@ -296,7 +391,7 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
 
 size_t gdn_wy_scratch_elems(int Hv, int dk, int dv, int T) {
     const size_t nblk = ((size_t)T + kC - 1) / kC;
-    return nblk * Hv * ((size_t)kC * dk + (size_t)kC * dv + (size_t)kC * kC + (size_t)dk * kC + kC);
+    return nblk * Hv * (3 * (size_t)kC * dk + (size_t)kC * dv + (size_t)kC * kC + kC);
 }
 
 // qn, kn [T, Hk, dk]; vv [T, Hv, dv]; lg, bg [T, Hv] (log decay, beta gate); o_raw [T, Hv*dv].
@@ -308,21 +403,22 @@ int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const fl
     const size_t nblk = ((size_t)T + kC - 1) / kC;
     if (nblk > 65535) return fail(MFA_ERR_SHAPE, "gdn blocked form: too many tokens in one call");
     const size_t slots = nblk * Hv;
-    float *Wc = scratch;
-    float *Uc = Wc + slots * kC * dk;
-    float *Mc = Uc + slots * kC * dv;
-    float *KdT = Mc + slots * kC * kC;
-    float *eLc = KdT + slots * dk * kC;
+    float *Wt = scratch;
+    float *Qt = Wt + slots * kC * dk;
+    float *Kt = Qt + slots * kC * dk;
+    float *Ut = Kt + slots * kC * dk;
+    float *Mt = Ut + slots * kC * dv;
+    float *eLc = Mt + slots * kC * kC;
     if (dk == 128) {
-        hipLaunchKernelGGL((gdn_wy_kernel<128>), dim3((unsigned)nblk, Hv), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
-                           lg, bg, Wc, Uc, Mc, KdT, eLc);
-        hipLaunchKernelGGL((gdn_wy_recur_kernel<128>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, qn, Wc, Uc,
-                           Mc, KdT, eLc, ssm, o_raw);
+        hipLaunchKernelGGL((gdn_wy_kernel<128>), dim3(Hv, (unsigned)nblk), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
+                           lg, bg, Wt, Qt, Ut, Mt, Kt, eLc);
+        hipLaunchKernelGGL((gdn_wy_recur_kernel<128>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, Wt, Qt, Ut,
+                           Mt, Kt, eLc, ssm, o_raw);
     } else {
-        hipLaunchKernelGGL((gdn_wy_kernel<64>), dim3((unsigned)nblk, Hv), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
-                           lg, bg, Wc, Uc, Mc, KdT, eLc);
-        hipLaunchKernelGGL((gdn_wy_recur_kernel<64>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, qn, Wc, Uc,
-                           Mc, KdT, eLc, ssm, o_raw);
+        hipLaunchKernelGGL((gdn_wy_kernel<64>), dim3(Hv, (unsigned)nblk), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
+                           lg, bg, Wt, Qt, Ut, Mt, Kt, eLc);
+        hipLaunchKernelGGL((gdn_wy_recur_kernel<64>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, Wt, Qt, Ut,
+                           Mt, Kt, eLc, ssm, o_raw);
     }
     MFA_HIP(hipGetLastError());
     return MFA_OK;
