@@ -20,62 +20,96 @@ namespace mfa {
 
 static constexpr int kSlab = 32;  // tokens staged in LDS at a time
 
-// grid (T, Hk + ceil(Hv*DV / 256) + 1), 256 threads.
-//   y <  Hk            : q and k channels of k-head y (conv, SiLU, norm, scaling)
+static constexpr int kPreTok = 8;  // tokens per workgroup of the first kernel
+
+// grid (ceil(T / 8), Hk + ceil(Hv*DV / 256) + 1), 256 threads; a workgroup serves 8 tokens.
+//   y <  Hk            : q and k channels of k-head y (conv, SiLU, norm, scaling, k^ . q^)
 //   Hk <= y < Hk + nvb : 256 v channels each (conv, SiLU)
 //   y == Hk + nvb      : decay and beta of every value head
 template <int DK>
 __global__ __launch_bounds__(256) void gdn_chunk_pre_kernel(
-    int Hk, int Hv, int DV, int K, int64_t step, const uint16_t *__restrict__ conv_w,
+    int Hk, int Hv, int DV, int K, int T, int step_mod, const uint16_t *__restrict__ conv_w,
     const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
     const float *__restrict__ ring, const float *__restrict__ qkv, const float *__restrict__ alpha,
     const float *__restrict__ beta, float *__restrict__ qn, float *__restrict__ kn,
     float *__restrict__ vv, float *__restrict__ gd, float *__restrict__ bg, float *__restrict__ kq,
     float *__restrict__ lg) {
     static_assert(2 * DK <= 256, "one workgroup covers a k-head's q and k channels");
-    __shared__ float s_part[4];
-    __shared__ float s_qk[2 * DK];
-    const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x;
+    constexpr int TT = kPreTok;
+    __shared__ float s_part[TT][4];
+    __shared__ float s_qk[TT][2 * DK];
+    const int t0 = blockIdx.x * TT, y = blockIdx.y, tid = threadIdx.x;
+    const int nt = T - t0 < TT ? T - t0 : TT;
     const int C = 2 * Hk * DK + Hv * DV;
     const int nvb = (Hv * DV + 255) / 256;
     if (y < Hk) {
         // threads [0, DK) are q channels, [DK, 2DK) are k channels of this head
         const bool act = tid < 2 * DK, is_q = tid < DK;
-        float c = 0.f;
-        if (act) {
-            const int ch = is_q ? y * DK + tid : Hk * DK + y * DK + (tid - DK);
-            c = conv_silu(ring, qkv, conv_w, C, K, step, t, ch);
-        }
-        const float ws = group_sum<64>(act ? c * c : 0.f);
-        if ((tid & 63) == 0) s_part[tid >> 6] = ws;
-        __syncthreads();
-        if (act) {
-            float sum = 0.f;
+        const int ch = is_q ? y * DK + tid : Hk * DK + y * DK + (tid - DK);
+        float c[TT];
 #pragma unroll
-            for (int w = 0; w < DK / 64; w++) sum += s_part[(is_q ? 0 : DK / 64) + w];
-            // infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2, k *= 1/sqrt(dk)
-            const float inv_rms = 1.0f / sqrtf(sum / (float)DK + 1e-6f);
-            const float inv_scale = 1.0f / sqrtf((float)DK);
-            float v = c * inv_rms;
-            v *= is_q ? inv_scale * inv_scale : inv_scale;
-            if (is_q) qn[((size_t)t * Hk + y) * DK + tid] = v;
-            else kn[((size_t)t * Hk + y) * DK + (tid - DK)] = v;
-            s_qk[tid] = v;
+        for (int i = 0; i < TT; i++) c[i] = 0.f;
+        if (act) {
+            if (K == 4) {
+                conv_silu_run<TT, 4>(ring, qkv, conv_w, C, step_mod, t0, nt, ch, c);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TT; i++)
+                    if (i < nt) c[i] = conv_silu(ring, qkv, conv_w, C, K, step_mod, t0 + i, ch);
+            }
         }
-        // k^ . q^ of the token, for the recurrence's read-out
+#pragma unroll
+        for (int i = 0; i < TT; i++) {
+            const float ws = group_sum<64>(c[i] * c[i]);
+            if ((tid & 63) == 0) s_part[i][tid >> 6] = ws;
+        }
         __syncthreads();
-        if (tid < 64) {
+        if (act) {
+            // infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2, k *= 1/sqrt(dk)
+            const float inv_scale = 1.0f / sqrtf((float)DK);
+#pragma unroll
+            for (int i = 0; i < TT; i++) {
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < DK / 64; w++) sum += s_part[i][(is_q ? 0 : DK / 64) + w];
+                const float inv_rms = 1.0f / sqrtf(sum / (float)DK + 1e-6f);
+                float v = c[i] * inv_rms;
+                v *= is_q ? inv_scale * inv_scale : inv_scale;
+                s_qk[i][tid] = v;
+                if (i < nt) {
+                    if (is_q) qn[((size_t)(t0 + i) * Hk + y) * DK + tid] = v;
+                    else kn[((size_t)(t0 + i) * Hk + y) * DK + (tid - DK)] = v;
+                }
+            }
+        }
+        // k^ . q^ of each token, for the read-out of the token-by-token recurrence
+        __syncthreads();
+        for (int i = tid >> 6; i < nt; i += 4) {
+            const int l = tid & 63;
             float d = 0.f;
 #pragma unroll
-            for (int i = 0; i < DK / 64; i++) d = fmaf(s_qk[tid + 64 * i], s_qk[DK + tid + 64 * i], d);
+            for (int u = 0; u < DK / 64; u++) d = fmaf(s_qk[i][l + 64 * u], s_qk[i][DK + l + 64 * u], d);
             d = group_sum<64>(d);
-            if (tid == 0) kq[(size_t)t * Hk + y] = d;
+            if (l == 0) kq[(size_t)(t0 + i) * Hk + y] = d;
         }
     } else if (y < Hk + nvb) {
         const int i = (y - Hk) * 256 + tid;
-        if (i < Hv * DV) vv[(size_t)t * Hv * DV + i] = conv_silu(ring, qkv, conv_w, C, K, step, t, 2 * Hk * DK + i);
+        if (i < Hv * DV) {
+            float c[TT];
+            if (K == 4) {
+                conv_silu_run<TT, 4>(ring, qkv, conv_w, C, step_mod, t0, nt, 2 * Hk * DK + i, c);
+            } else {
+#pragma unroll
+                for (int u = 0; u < TT; u++)
+                    c[u] = u < nt ? conv_silu(ring, qkv, conv_w, C, K, step_mod, t0 + u, 2 * Hk * DK + i) : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < TT; u++)
+                if (u < nt) vv[(size_t)(t0 + u) * Hv * DV + i] = c[u];
+        }
     } else {
-        for (int h = tid; h < Hv; h += 256) {
+        for (int p = tid; p < nt * Hv; p += 256) {
+            const int t = t0 + p / Hv, h = p % Hv;
             // shaders.metal:1321-1326
             const float a_cap = expf(a_log[h]);
             const float sp = logf(1.0f + expf(alpha[(size_t)t * Hv + h] + bf16_bits_to_f32(dt_bias[h])));
@@ -185,33 +219,36 @@ __global__ __launch_bounds__(256) void gdn_chunk_recur_kernel(
     for (int i = 0; i < NI; i++) *(float4 *)(srow + 64 * i) = s[i];
 }
 
-// grid (T, Hv) for the gated norm (shaders.metal:1337-1370) plus, at x == T, blocks that
-// advance the conv ring: input number s lives in slot s % K, so the last min(T, K)
-// inputs of the chunk overwrite their slots.
-__global__ __launch_bounds__(128) void gdn_chunk_post_kernel(
-    int Hv, int DV, int T, int C, int K, int64_t step, float eps, const float *__restrict__ o_raw,
+// The gated norm (shaders.metal:1337-1370), one wave per (token, head) pair, four pairs per
+// workgroup, in blocks [0, npb); blocks [npb, npb + 32) advance the conv ring: input number s
+// lives in slot s % K, so the last min(T, K) inputs of the chunk overwrite their slots.
+__global__ __launch_bounds__(256) void gdn_chunk_post_kernel(
+    int Hv, int DV, int T, int C, int K, int64_t step, float eps, int npb, const float *__restrict__ o_raw,
     const float *__restrict__ z, const uint16_t *__restrict__ norm_w, const float *__restrict__ qkv,
     float *__restrict__ ring, float *__restrict__ out) {
-    __shared__ float s_part[2];
     const int tid = threadIdx.x;
-    if ((int)blockIdx.x == T) {
-        const int first = T > K ? T - K : 0;
+    if ((int)blockIdx.x >= npb) {
+        const int first = T > K ? T - K : 0, nb = gridDim.x - npb;
         for (int t = first; t < T; t++) {
             const int slot = (int)((step + t) % K);
-            for (int ch = blockIdx.y * 128 + tid; ch < C; ch += gridDim.y * 128)
+            for (int ch = (blockIdx.x - npb) * 256 + tid; ch < C; ch += nb * 256)
                 ring[(size_t)slot * C + ch] = qkv[(size_t)t * C + ch];
         }
         return;
     }
-    const size_t base = ((size_t)blockIdx.x * Hv + blockIdx.y) * DV;
-    float sq = 0.f;
-    for (int i = tid; i < DV; i += 128) sq += o_raw[base + i] * o_raw[base + i];
-    const float ws = group_sum<64>(sq);
-    if ((tid & 63) == 0) s_part[tid >> 6] = ws;
-    __syncthreads();
-    const float inv = 1.0f / sqrtf((s_part[0] + s_part[1]) / (float)DV + eps);
-    for (int i = tid; i < DV; i += 128)
-        out[base + i] = o_raw[base + i] * inv * bf16_bits_to_f32(norm_w[i]) * silu_f(z[base + i]);
+    const int64_t pair = (int64_t)blockIdx.x * 4 + (tid >> 6);
+    if (pair >= (int64_t)T * Hv) return;
+    const int lane = tid & 63;
+    const size_t base = (size_t)pair * DV;
+    // lane l holds elements l and l + 64; the two halves are summed separately and then
+    // added, the order of the single-step kernel's norm
+    const float x0 = lane < DV ? o_raw[base + lane] : 0.f;
+    const float x1 = lane + 64 < DV ? o_raw[base + lane + 64] : 0.f;
+    const float sum = group_sum<64>(x0 * x0) + group_sum<64>(x1 * x1);
+    const float inv = 1.0f / sqrtf(sum / (float)DV + eps);
+    if (lane < DV) out[base + lane] = x0 * inv * bf16_bits_to_f32(norm_w[lane]) * silu_f(z[base + lane]);
+    if (lane + 64 < DV)
+        out[base + lane + 64] = x1 * inv * bf16_bits_to_f32(norm_w[lane + 64]) * silu_f(z[base + lane + 64]);
 }
 
 // Chunks of at least this many tokens take the blocked form on the matrix cores; shorter
@@ -248,12 +285,12 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
     const int nvb = (Hv * dv + 255) / 256;
     const bool blocked = T >= kWyMinTokens;
     if (dk == 128)
-        hipLaunchKernelGGL((gdn_chunk_pre_kernel<128>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
-                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
+        hipLaunchKernelGGL((gdn_chunk_pre_kernel<128>), dim3((T + kPreTok - 1) / kPreTok, Hk + nvb + 1), dim3(256), 0, s,
+                           Hk, Hv, dv, K, T, (int)(step % K), w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
                            vv, gd, bg, kq, lg);
     else
-        hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3(T, Hk + nvb + 1), dim3(256), 0, s, Hk, Hv, dv,
-                           K, step, w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
+        hipLaunchKernelGGL((gdn_chunk_pre_kernel<64>), dim3((T + kPreTok - 1) / kPreTok, Hk + nvb + 1), dim3(256), 0, s,
+                           Hk, Hv, dv, K, T, (int)(step % K), w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
                            vv, gd, bg, kq, lg);
     MFA_HIP(hipGetLastError());
     if (blocked) {
@@ -266,7 +303,8 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
                            vv, gd, bg, kq, ssm, o_raw);
     }
     MFA_HIP(hipGetLastError());
-    hipLaunchKernelGGL(gdn_chunk_post_kernel, dim3(T + 1, Hv), dim3(128), 0, s, Hv, dv, T, C, K, step, eps,
+    const int npb = (int)(((int64_t)T * Hv + 3) / 4);
+    hipLaunchKernelGGL(gdn_chunk_post_kernel, dim3(npb + 32), dim3(256), 0, s, Hv, dv, T, C, K, step, eps, npb,
                        o_raw, z, w.norm_w, qkv_in, conv_ring, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;

@@ -109,19 +109,49 @@ __device__ inline float delta_row16(float4 (&s)[DK / 64], const float4 (&kk)[DK 
     return fmaf(delta, kq, g * sq);
 }
 
-// Depthwise conv + SiLU of channel ch for the input numbered `step + t` of the layer
-// (crates/moeflux/src/riir/linear_attn.rs:132-154): tap k < K-1 multiplies input
-// step+t-(K-1)+k, which is row t-(K-1)+k of `chunk` when that is >= 0 and the ring slot
-// (input number mod K) of the history otherwise; tap K-1 multiplies the new input.
+// Depthwise conv + SiLU of channel ch for TT consecutive inputs of the layer, the first
+// of them input number `step + t0` (crates/moeflux/src/riir/linear_attn.rs:132-154): tap
+// k < K-1 of token t multiplies input step+t-(K-1)+k, which is row t-(K-1)+k of `chunk`
+// when that is >= 0 and the ring slot (input number mod K) of the history otherwise; tap
+// K-1 multiplies the new input.  Tokens at or past nt give 0.  step_mod = step % K.
+// Each input is loaded once and the taps stay in registers.
+template <int TT, int KC>
+__device__ inline void conv_silu_run(const float *__restrict__ ring, const float *__restrict__ chunk,
+                                     const uint16_t *__restrict__ w, int C, int step_mod, int t0, int nt,
+                                     int ch, float (&out)[TT]) {
+    float wt[KC], xs[TT + KC - 1];
+#pragma unroll
+    for (int k = 0; k < KC; k++) wt[k] = bf16_bits_to_f32(w[(size_t)ch * KC + k]);
+#pragma unroll
+    for (int j = 0; j < TT + KC - 1; j++) {
+        const int idx = t0 - (KC - 1) + j;  // row of the chunk, negative: history
+        float x = 0.f;
+        if (idx >= 0) {
+            if (idx < t0 + nt) x = chunk[(size_t)idx * C + ch];
+        } else {
+            x = ring[(size_t)(((step_mod + idx) % KC + KC) % KC) * C + ch];
+        }
+        xs[j] = x;
+    }
+#pragma unroll
+    for (int i = 0; i < TT; i++) {
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < KC; k++) acc = fmaf(xs[i + k], wt[k], acc);
+        out[i] = i < nt ? silu_f(acc) : 0.f;
+    }
+}
+
+// The same for a conv width known only at run time, one token at a time.
 __device__ inline float conv_silu(const float *__restrict__ ring, const float *__restrict__ chunk,
-                                  const uint16_t *__restrict__ w, int C, int K, int64_t step, int t,
+                                  const uint16_t *__restrict__ w, int C, int K, int step_mod, int t,
                                   int ch) {
     float acc = 0.f;
     for (int k = 0; k < K - 1; k++) {
         const int idx = t - (K - 1) + k;
         float x;
         if (idx >= 0) x = chunk[(size_t)idx * C + ch];
-        else x = ring[(size_t)(((step + idx) % K + K) % K) * C + ch];
+        else x = ring[(size_t)(((step_mod + idx) % K + K) % K) * C + ch];
         acc = fmaf(x, bf16_bits_to_f32(w[(size_t)ch * K + k]), acc);
     }
     acc = fmaf(chunk[(size_t)t * C + ch], bf16_bits_to_f32(w[(size_t)ch * K + (K - 1)]), acc);
