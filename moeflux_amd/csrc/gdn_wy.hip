@@ -38,20 +38,6 @@ __device__ inline wy_f32x4 mfma4(float4 a, float4 b, wy_f32x4 acc) {
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
     return acc;
 }
-// The same four instructions on four accumulators: a dependent v_mfma has to wait for the
-// previous one to leave the pipeline, about three times its issue time, so long
-// contractions keep four independent chains going and add them at the end.
-struct Acc4 {
-    wy_f32x4 a[4];
-    __device__ Acc4() { a[0] = a[1] = a[2] = a[3] = wy_f32x4{0.f, 0.f, 0.f, 0.f}; }
-    __device__ wy_f32x4 sum() const { return (a[0] + a[1]) + (a[2] + a[3]); }
-};
-__device__ inline void mfma4x(float4 a, float4 b, Acc4 &acc) {
-    acc.a[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc.a[0], 0, 0, 0);
-    acc.a[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc.a[1], 0, 0, 0);
-    acc.a[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc.a[2], 0, 0, 0);
-    acc.a[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc.a[3], 0, 0, 0);
-}
 __device__ inline float4 lds_f4(const float *p) {
     const gdn_f32x4 v = *reinterpret_cast<const gdn_f32x4 *>(p);
     return float4{v.x, v.y, v.z, v.w};
@@ -86,7 +72,7 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     __shared__ __align__(16) float sQ[kC][LDK];  // q^, later v
     __shared__ __align__(16) float sA[kC][LDC];
     __shared__ __align__(16) float sT[kC][LDC];
-    __shared__ __align__(16) float sL[kC], sB[kC], sCw[kC];
+    __shared__ __align__(16) float sL[kC], sB[kC], sCw[kC], sKd[kC];
 
     // heads along x: a head's blocks are produced on the XCD whose L2 the recurrence kernel
     // (heads along x as well) will read them through
@@ -98,16 +84,24 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     const size_t slot = (size_t)blk * Hv + vh;
 
     // ---- phase 0: k^, q^ of the block, cumulative log decay, beta ---------------------
-    for (int i = tid; i < kC * (DK / 4); i += 256) {
-        const int tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
-        float4 a = {0.f, 0.f, 0.f, 0.f}, b = a;
-        if (tt < nt) {
-            const size_t src = ((size_t)(t0 + tt) * Hk + kh) * DK + x;
-            a = load_f4(kn + src);
-            b = load_f4(qn + src);
+    {
+        // all of a thread's requests go out before the first of them is stored
+        constexpr int NL = kC * (DK / 4) / 256;
+        float4 a[NL], b[NL];
+#pragma unroll
+        for (int u = 0; u < NL; u++) {
+            const int i = tid + u * 256, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
+            const size_t src = ((size_t)(t0 + (tt < nt ? tt : nt - 1)) * Hk + kh) * DK + x;
+            a[u] = load_f4(kn + src);
+            b[u] = load_f4(qn + src);
         }
-        *(float4 *)&sK[tt][x] = a;
-        *(float4 *)&sQ[tt][x] = b;
+#pragma unroll
+        for (int u = 0; u < NL; u++) {
+            const int i = tid + u * 256, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
+            const float keep = tt < nt ? 1.f : 0.f;  // padded tokens are zero rows
+            *(float4 *)&sK[tt][x] = float4{a[u].x * keep, a[u].y * keep, a[u].z * keep, a[u].w * keep};
+            *(float4 *)&sQ[tt][x] = float4{b[u].x * keep, b[u].y * keep, b[u].z * keep, b[u].w * keep};
+        }
     }
     if (wave == 0) {
         float l = lane < nt ? lg[(size_t)(t0 + lane) * Hv + vh] : 0.f;
@@ -121,29 +115,29 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
         sB[lane] = b;
         sCw[lane] = b * expf(l);
         eLc[slot * kC + lane] = expf(l);
+        sKd[lane] = expf(__shfl(l, 63, 64) - l);  // e^{L_C - L_t}
     }
     __syncthreads();
 
     // ---- phase 1: the lower tiles of K K^T (-> A) and of Q K^T (-> M) -----------------
     // 10 tiles (I, J <= I) each; 20 jobs of DK/4 instructions over 4 waves.
-#pragma unroll 1
+#pragma unroll
     for (int r = 0; r < 5; r++) {
         const int job = wave * 5 + r, kind = job / 10, idx = job % 10;
         const int I = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
         const int J = idx - I * (I + 1) / 2;
         const float(*X)[LDK] = kind ? sQ : sK;
-        Acc4 acc4;
+        wy_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < DK / 16; s++)
-            mfma4x(lds_f4(&X[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc4);
-        const wy_f32x4 acc = acc4.sum();
+            acc = mfma4(lds_f4(&X[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc);
         // lane (n = m, g) holds rows 16I + 4g + i of column 16J + n
         const int col = 16 * J + m;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int row = 16 * I + 4 * g + i;
             const float dl = sL[row] - sL[col];
-            const float d = expf(dl < 0.f ? dl : 0.f);
+            const float d = __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);  // v_exp_f32: 1 ulp
             if (kind == 0) sA[row][col] = (col < row) ? sB[row] * d * acc[i] : 0.f;
             else  // to tile (I, J) in A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
                 Mt[((slot * 4 + I) * 4 + J) * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = (col <= row) ? d * acc[i] : 0.f;
@@ -160,22 +154,26 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     //      per wave, a column per lane), the blocks below them level by level from
     //      T_IJ = -T_II sum_{J <= K < I} A_IK T_KJ on the matrix cores -----------------------
     {
-        const float lc = sL[kC - 1];
-        for (int i = tid; i < NK * 4 * 64; i += 256) {
-            const int tile = i >> 6, l = i & 63, c = tile >> 2, tau = tile & 3;
+        constexpr int NL = kC * (DV / 4) / 256;
+        float4 a[NL];
+#pragma unroll
+        for (int u = 0; u < NL; u++) {
+            const int i = tid + u * 256, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
+            a[u] = load_f4(vv + ((size_t)(t0 + (tt < nt ? tt : nt - 1)) * Hv + vh) * DV + x);
+        }
+#pragma unroll
+        for (int u = 0; u < NK * 4 * 64 / 256; u++) {
+            const int i = tid + u * 256, tile = i >> 6, l = i & 63, c = tile >> 2, tau = tile & 3;
             const int kk = 16 * c + (l & 15), j4 = 16 * tau + 4 * (l >> 4);
-            float4 o;
-            o.x = expf(lc - sL[j4 + 0]) * sK[j4 + 0][kk];
-            o.y = expf(lc - sL[j4 + 1]) * sK[j4 + 1][kk];
-            o.z = expf(lc - sL[j4 + 2]) * sK[j4 + 2][kk];
-            o.w = expf(lc - sL[j4 + 3]) * sK[j4 + 3][kk];
+            const float4 e = lds_f4(&sKd[j4]);
+            const float4 o = {e.x * sK[j4 + 0][kk], e.y * sK[j4 + 1][kk], e.z * sK[j4 + 2][kk], e.w * sK[j4 + 3][kk]};
             *(float4 *)(Kt + (slot * NK * 4 + tile) * 256 + l * 4) = o;
         }
-        for (int i = tid; i < kC * (DV / 4); i += 256) {
-            const int tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
-            float4 a = {0.f, 0.f, 0.f, 0.f};
-            if (tt < nt) a = load_f4(vv + ((size_t)(t0 + tt) * Hv + vh) * DV + x);
-            *(float4 *)&sQ[tt][x] = a;
+#pragma unroll
+        for (int u = 0; u < NL; u++) {
+            const int i = tid + u * 256, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
+            const float keep = tt < nt ? 1.f : 0.f;
+            *(float4 *)&sQ[tt][x] = float4{a[u].x * keep, a[u].y * keep, a[u].z * keep, a[u].w * keep};
         }
     }
     {
@@ -235,7 +233,9 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
             }
 #pragma unroll
     for (int tau = 0; tau < 4; tau++) {
-        Acc4 aw4[NCT], au4[NCT];
+        wy_f32x4 aw4[NCT], au4[NCT];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ct++) aw4[ct] = au4[ct] = wy_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s <= tau; s++) {
             const float4 t4 = lds_f4(&sT[16 * tau + m][16 * s + 4 * g]);
@@ -244,13 +244,13 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
             const float4 tu = {t4.x * cb.x, t4.y * cb.y, t4.z * cb.z, t4.w * cb.w};
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) {
-                mfma4x(tw, float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, aw4[ct]);
-                mfma4x(tu, float4{bV[s][ct][0], bV[s][ct][1], bV[s][ct][2], bV[s][ct][3]}, au4[ct]);
+                aw4[ct] = mfma4(tw, float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, aw4[ct]);
+                au4[ct] = mfma4(tu, float4{bV[s][ct][0], bV[s][ct][1], bV[s][ct][2], bV[s][ct][3]}, au4[ct]);
             }
         }
 #pragma unroll
         for (int ct = 0; ct < NCT; ct++) {
-            const wy_f32x4 aw = aw4[ct].sum(), au = au4[ct].sum();
+            const wy_f32x4 aw = aw4[ct], au = au4[ct];
             const size_t tile = (slot * 4 + tau) * NK + NCT * wave + ct;
             // U as computed; W to A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
             *reinterpret_cast<wy_f32x4 *>(Ut + tile * 256 + lane * 4) = au;
@@ -325,13 +325,12 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
     auto block = [&](int blk, const Late &cur, Late &nxt) __attribute__((always_inline)) {
         const int t0 = blk * kC;
         // ---- W S0^T and Q S0^T for this wave's 16 tokens ------------------------------
-        Acc4 p1x, p2x;
+        wy_f32x4 p1 = {0.f, 0.f, 0.f, 0.f}, p2 = p1;
 #pragma unroll
         for (int c = 0; c < NK; c++) {
-            mfma4x(pw[c], as_f4(st[c]), p1x);
-            mfma4x(pq[c], as_f4(st[c]), p2x);
+            p1 = mfma4(pw[c], as_f4(st[c]), p1);
+            p2 = mfma4(pq[c], as_f4(st[c]), p2);
         }
-        const wy_f32x4 p1 = p1x.sum(), p2 = p2x.sum();
         fetch_wq(blk + 1);
         // ---- D = U - W S0^T: lane (n, g) holds tokens 16w+4g+i of state row row0+n ----
         wy_f32x4 d;
@@ -341,11 +340,10 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
         s_d[wave][lane] = d;
         __syncthreads();
         // ---- O = diag(e^L) Q S0^T + M D ------------------------------------------------
-        Acc4 ox;
+        wy_f32x4 o = cur.el * p2;
 #pragma unroll
         for (int tau = 0; tau < 4; tau++)
-            if (tau <= wave) mfma4x(as_f4(cur.mt[tau]), as_f4(s_d[tau][lane]), ox);
-        const wy_f32x4 o = cur.el * p2 + ox.sum();
+            if (tau <= wave) o = mfma4(as_f4(cur.mt[tau]), as_f4(s_d[tau][lane]), o);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int t = t0 + 16 * wave + 4 * g + i;
@@ -358,10 +356,11 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
 #pragma unroll
             for (int kt = 0; kt < NKW; kt++) {
                 constexpr int c0 = NKW * w;
-                Acc4 ux;
+                wy_f32x4 acc = st[c0 + kt] * cur.elc;
 #pragma unroll
-                for (int tau = 0; tau < 4; tau++) mfma4x(as_f4(cur.kd[kt][tau]), as_f4(s_d[tau][lane]), ux);
-                s_st[c0 + kt][lane] = st[c0 + kt] * cur.elc + ux.sum();
+                for (int tau = 0; tau < 4; tau++)
+                    acc = mfma4(as_f4(cur.kd[kt][tau]), as_f4(s_d[tau][lane]), acc);
+                s_st[c0 + kt][lane] = acc;
             }
         };
         if (wave == 0) update(std::integral_constant<int, 0>{});
