@@ -14,7 +14,10 @@ fn main() {
     cmd.args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-ffp-contract=off"])
         .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"])
         .arg("-I").arg(root.join("include")).arg("-I").arg(&csrc);
-    for f in ["api.hip", "sdpa_decode.hip", "attn_kernels.hip", "gdn.hip"] {
+    for f in [
+        "api.hip", "kv_cache.hip", "sdpa_decode.hip", "sdpa_prefill.hip", "attn_kernels.hip", "gdn.hip",
+        "gdn_chunk.hip", "gdn_wy.hip",
+    ] {
         println!("cargo:rerun-if-changed=csrc/{f}");
         cmd.arg(csrc.join(f));
     }
