@@ -123,6 +123,38 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
 int mfa_sdpa_decode_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev,
                         const float *q_gate_dev, float *out_dev);
 
+/* ---- what precedes the attention core in a full-attention layer -------------- */
+
+/* Per-layer constants of the prologue: the bf16 weights of the per-head RMS
+ * norms of q and k (model.layers.N.self_attn.{q,k}_norm.weight,
+ * full_attn_forward.rs:256-277), head_dim values each. */
+int mfa_set_full_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *q_norm_bf16,
+                         const uint16_t *k_norm_bf16);
+/* The rotation of q and k: base frequency and number of rotated channels per
+ * head.  Defaults at create: theta = 1e7, rotary_dim = head_dim / 4
+ * (variants.rs:245-250, 369). */
+int mfa_set_rope(mfa_ctx *ctx, float theta, int32_t rotary_dim);
+
+/* Replaces the host round trip of full_attn_forward.rs:234-323 for one token:
+ * the q projection's output [Hq][q_h | gate_h] is split (238-254), q and k get
+ * the per-head RMS norm (rms_norm.rs:104-156), the first rotary_dim channels of
+ * every q and k head are rotated at position `pos` (rope.rs:65-131), and k
+ * (normed, rotated) and v (as is) are appended to the layer's cache
+ * (282-323).  q_out, q_gate_out: [Hq*head_dim], what mfa_sdpa_decode takes.
+ * MFA_ERR_OVERFLOW when the layer is full. */
+int mfa_attn_prologue(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out,
+                      const float *k, const float *v, float *q_out, float *q_gate_out);
+int mfa_attn_prologue_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
+                          const float *k_dev, const float *v_dev, float *q_out_dev,
+                          float *q_gate_out_dev);
+/* The prologue followed by the attention core on the appended cache: everything
+ * of full_attn_layer_forward between the projections and o_proj
+ * (full_attn_forward.rs:234-389).  out: [Hq*head_dim]. */
+int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out,
+                       const float *k, const float *v, float *out);
+int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
+                           const float *k_dev, const float *v_dev, float *out_dev);
+
 /* A chunk of T prompt tokens on one full-attention layer.  The reference has
  * no batched prefill: eval_prompt is a token loop (riir/mod.rs:1196-1214); the
  * result equals T successive mfa_kv_append + mfa_sdpa_decode calls.

@@ -100,6 +100,20 @@ static int slab_alloc(Ctx *c, size_t bytes, char **out) {
     return MFA_OK;
 }
 
+// The frequency table of rope.rs:99-103, with the host's powf (the reference computes the
+// same expression with its libm on every call), uploaded once.
+static int set_rope(Ctx *c, float theta, int32_t rotary_dim) {
+    if (!c->inv_freq) return fail(MFA_ERR_LAYER, "the context has no full-attention layer");
+    if (!(theta > 0.f) || rotary_dim <= 0 || rotary_dim > c->cfg.head_dim || (rotary_dim & 1))
+        return fail(MFA_ERR_INVALID, "rope: theta %g, rotary_dim %d (even, in (0, head_dim])", (double)theta, rotary_dim);
+    std::vector<float> f((size_t)rotary_dim / 2);
+    for (int i = 0; i < rotary_dim / 2; i++) f[i] = 1.0f / powf(theta, (float)(2 * i) / (float)rotary_dim);
+    MFA_HIP(hipMemcpyAsync(c->inv_freq, f.data(), f.size() * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    c->rotary_dim = rotary_dim;
+    return MFA_OK;
+}
+
 static int validate(const mfa_config *cfg, bool *has_full, bool *has_lin) {
     if (!cfg) return fail(MFA_ERR_INVALID, "NULL config");
     if (cfg->num_layers <= 0 || cfg->full_attn_interval <= 0)
@@ -174,10 +188,22 @@ static int create(const mfa_config *cfg, Ctx **out) {
         char *kslab, *vslab;
         MFA_TRY(slab_alloc(c, bytes * nfull, &kslab));
         MFA_TRY(slab_alloc(c, bytes * nfull, &vslab));
+        char *norms;
+        MFA_TRY(slab_alloc(c, (size_t)nfull * 2 * cfg->head_dim * 2, &norms));
         for (int i = 0; i < nfull; i++) {
             c->full[i].k = kslab + (size_t)i * bytes;
             c->full[i].v = vslab + (size_t)i * bytes;
+            c->full[i].q_norm = (uint16_t *)norms + (size_t)(2 * i) * cfg->head_dim;
+            c->full[i].k_norm = (uint16_t *)norms + (size_t)(2 * i + 1) * cfg->head_dim;
         }
+        char *rope;
+        MFA_TRY(slab_alloc(c, (size_t)cfg->head_dim * sizeof(float), &rope));
+        c->inv_freq = (float *)rope;
+        char *qg;
+        MFA_TRY(slab_alloc(c, 2 * (size_t)cfg->num_attn_heads * cfg->head_dim * sizeof(float), &qg));
+        c->qg_stage = (float *)qg;
+        // variants.rs:245-250, 369: a quarter of the head is rotated, theta = 1e7
+        MFA_TRY(set_rope(c, 1.0e7f, cfg->head_dim / 4));
         int splits = sdpa_pick_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
                                       cfg->head_dim, cfg->kv_capacity, c->num_cus, 0);
         if (splits < 128) splits = 128;
@@ -434,6 +460,24 @@ int mfa_set_partial_only(mfa_ctx *ctx, int32_t on) {
     return MFA_OK;
 }
 
+int mfa_set_full_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_norm_bf16 || !k_norm_bf16) return fail(MFA_ERR_INVALID, "NULL weight pointer");
+    MFA_TRY(h2d(c, f->q_norm, q_norm_bf16, (size_t)c->cfg.head_dim * 2));
+    MFA_TRY(h2d(c, f->k_norm, k_norm_bf16, (size_t)c->cfg.head_dim * 2));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    f->norms_set = true;
+    return MFA_OK;
+}
+
+int mfa_set_rope(mfa_ctx *ctx, float theta, int32_t rotary_dim) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    return set_rope(c, theta, rotary_dim);
+}
+
 /* ---- full attention -------------------------------------------------------- */
 
 int mfa_kv_append_dev(mfa_ctx *ctx, int32_t layer, const float *k_dev, const float *v_dev) {
@@ -487,6 +531,73 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
     MFA_TRY(h2d(c, c->stage + qd, q_gate, qd * 4));
     MFA_TRY(sdpa_decode_dev(c, f, c->stage, c->stage + qd, c->stage + 2 * qd));
     return d2h_sync(c, out, c->stage + 2 * qd, qd * 4);
+}
+
+static int prologue_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_proj, const float *k, const float *v,
+                        float *q_out, float *gate_out) {
+    if (!f->norms_set) return fail(MFA_ERR_INVALID, "q/k norm weights not set (mfa_set_full_weights)");
+    if ((int64_t)f->len + 1 > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + 1 > capacity %d", f->len, c->cfg.kv_capacity);
+    MFA_TRY(launch_attn_prologue(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
+                                 c->cfg.head_dim, c->rotary_dim, c->cfg.rms_norm_eps, pos, f->len, c->plane_elems,
+                                 f->q_norm, f->k_norm, c->inv_freq, q_proj, k, v, q_out, gate_out, f->k, f->v));
+    f->len += 1;
+    return MFA_OK;
+}
+
+int mfa_attn_prologue_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
+                          const float *k_dev, const float *v_dev, float *q_out_dev, float *q_gate_out_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out_dev || !k_dev || !v_dev || !q_out_dev || !q_gate_out_dev)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    return prologue_dev(c, f, pos, q_proj_out_dev, k_dev, v_dev, q_out_dev, q_gate_out_dev);
+}
+
+int mfa_attn_prologue(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out, const float *k,
+                      const float *v, float *q_out, float *q_gate_out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out || !k || !v || !q_out || !q_gate_out) return fail(MFA_ERR_INVALID, "NULL argument");
+    const size_t qd = (size_t)c->q_dim(), kd = (size_t)c->kv_dim();
+    MFA_TRY(ensure_stage(c, 4 * qd + 2 * kd));
+    float *qp = c->stage, *kk = qp + 2 * qd, *vv = kk + kd, *qo = vv + kd, *go = qo + qd;
+    MFA_TRY(h2d(c, qp, q_proj_out, 2 * qd * 4));
+    MFA_TRY(h2d(c, kk, k, kd * 4));
+    MFA_TRY(h2d(c, vv, v, kd * 4));
+    MFA_TRY(prologue_dev(c, f, pos, qp, kk, vv, qo, go));
+    MFA_HIP(hipMemcpyAsync(q_out, qo, qd * 4, hipMemcpyDeviceToHost, c->stream));
+    return d2h_sync(c, q_gate_out, go, qd * 4);
+}
+
+int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
+                           const float *k_dev, const float *v_dev, float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out_dev || !k_dev || !v_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    const size_t qd = (size_t)c->q_dim();
+    MFA_TRY(prologue_dev(c, f, pos, q_proj_out_dev, k_dev, v_dev, c->qg_stage, c->qg_stage + qd));
+    return sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, out_dev);
+}
+
+int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out, const float *k,
+                       const float *v, float *out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out || !k || !v || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    const size_t qd = (size_t)c->q_dim(), kd = (size_t)c->kv_dim();
+    MFA_TRY(ensure_stage(c, 3 * qd + 2 * kd));
+    float *qp = c->stage, *kk = qp + 2 * qd, *vv = kk + kd, *oo = vv + kd;
+    MFA_TRY(h2d(c, qp, q_proj_out, 2 * qd * 4));
+    MFA_TRY(h2d(c, kk, k, kd * 4));
+    MFA_TRY(h2d(c, vv, v, kd * 4));
+    MFA_TRY(prologue_dev(c, f, pos, qp, kk, vv, c->qg_stage, c->qg_stage + qd));
+    MFA_TRY(sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, oo));
+    return d2h_sync(c, out, oo, qd * 4);
 }
 
 int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_dev,

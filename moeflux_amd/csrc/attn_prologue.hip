@@ -1,0 +1,91 @@
+// What a full-attention layer does between its q/k/v projections and the attention
+// core, as one launch on the device.
+//
+// The reference reads the three projection outputs back to the host and, per token,
+// splits the q projection into q and its output gate, applies the per-head RMS norm to
+// q and k, rotates the first rotary_dim channels of every q and k head, appends k and v
+// to the layer's cache and mirrors the row to the GPU
+// (crates/moeflux/src/riir/full_attn_forward.rs:238-323; rms_norm.rs:104-156;
+// rope.rs:65-131).  Here the projection outputs stay on the device: one workgroup per
+// q head, k head and v head does the same arithmetic and writes q, the gate and the
+// cache row (in the cache's tiled layout) directly.
+#include "gdn_device.h"
+
+namespace mfa {
+
+// f32 -> cache element
+template <typename KV> __device__ inline KV to_kv(float x);
+template <> __device__ inline float to_kv<float>(float x) { return x; }
+template <> __device__ inline uint16_t to_kv<uint16_t>(float x) { return f32_to_bf16_bits(x); }
+
+// grid Hq + 2*Hkv workgroups of D threads (D = 64, 128 or 256):
+//   [0, Hq)           q head: split off the gate, norm, rotate
+//   [Hq, Hq+Hkv)      k head: norm, rotate, store at cache position `cache_pos`
+//   [Hq+Hkv, Hq+2Hkv) v head: store at cache position `cache_pos`
+// q_proj: [Hq][2][D] (q_h then gate_h, full_attn_forward.rs:240-254).  inv_freq: the table
+// 1 / theta^(2i/rotary_dim), i < rotary_dim/2, computed on the host.
+template <typename KV>
+__global__ void attn_prologue_kernel(int Hq, int Hkv, int D, int rotary_dim, float eps, int32_t pos,
+                                     int64_t cache_pos, size_t plane_elems,
+                                     const uint16_t *__restrict__ q_norm, const uint16_t *__restrict__ k_norm,
+                                     const float *__restrict__ inv_freq, const float *__restrict__ q_proj,
+                                     const float *__restrict__ k_in, const float *__restrict__ v_in,
+                                     float *__restrict__ q_out, float *__restrict__ gate_out,
+                                     KV *__restrict__ k_tiled, KV *__restrict__ v_tiled) {
+    __shared__ float s_y[256];
+    __shared__ float s_part[4];
+    const int b = blockIdx.x, x = threadIdx.x;
+    if (b >= Hq + Hkv) {  // v is cached as it comes
+        const int kvh = b - Hq - Hkv;
+        v_tiled[(size_t)kvh * plane_elems + KvTile<KV>::v_off(cache_pos, x, D)] = to_kv<KV>(v_in[(size_t)kvh * D + x]);
+        return;
+    }
+    const bool is_q = b < Hq;
+    const int h = is_q ? b : b - Hq;
+    const float v = is_q ? q_proj[(size_t)h * 2 * D + x] : k_in[(size_t)h * D + x];
+    if (is_q) gate_out[(size_t)h * D + x] = q_proj[(size_t)h * 2 * D + D + x];
+    // per-head RMS norm: x * inv_rms * weight (rms_norm.rs:138-151)
+    const float ws = group_sum<64>(v * v);
+    if ((x & 63) == 0) s_part[x >> 6] = ws;
+    __syncthreads();
+    float sum = 0.f;
+    for (int w = 0; w < D / 64; w++) sum += s_part[w];
+    const float inv_rms = 1.0f / sqrtf(sum / (float)D + eps);
+    const float y = v * inv_rms * bf16_bits_to_f32((is_q ? q_norm : k_norm)[x]);
+    s_y[x] = y;
+    __syncthreads();
+    // rotation of the pairs (i, i + half), i < half = rotary_dim / 2 (rope.rs:96-112)
+    const int half = rotary_dim >> 1;
+    float r = y;
+    if (x < rotary_dim) {
+        const int i = x < half ? x : x - half;
+        const float angle = (float)pos * inv_freq[i];
+        const float cos_a = cosf(angle), sin_a = sinf(angle);
+        const float x0 = s_y[i], x1 = s_y[i + half];
+        r = x < half ? x0 * cos_a - x1 * sin_a : x0 * sin_a + x1 * cos_a;
+    }
+    if (is_q) q_out[(size_t)h * D + x] = r;
+    else k_tiled[(size_t)h * plane_elems + KvTile<KV>::k_off(cache_pos, x, D)] = to_kv<KV>(r);
+}
+
+int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
+                         int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,
+                         const uint16_t *k_norm, const float *inv_freq, const float *q_proj, const float *k_in,
+                         const float *v_in, float *q_out, float *gate_out, void *k_tiled, void *v_tiled) {
+    if (D != 64 && D != 128 && D != 256) return fail(MFA_ERR_SHAPE, "attention prologue: head_dim %d not supported", D);
+    if (rotary_dim <= 0 || rotary_dim > D || (rotary_dim & 1))
+        return fail(MFA_ERR_INVALID, "attention prologue: rotary_dim %d must be even and in (0, head_dim]", rotary_dim);
+    if (pos < 0) return fail(MFA_ERR_INVALID, "attention prologue: pos %d < 0", pos);
+    if (kv_dtype == MFA_KV_BF16)
+        hipLaunchKernelGGL((attn_prologue_kernel<uint16_t>), dim3(Hq + 2 * Hkv), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
+                           eps, pos, cache_pos, plane_elems, q_norm, k_norm, inv_freq, q_proj, k_in, v_in, q_out,
+                           gate_out, (uint16_t *)k_tiled, (uint16_t *)v_tiled);
+    else
+        hipLaunchKernelGGL((attn_prologue_kernel<float>), dim3(Hq + 2 * Hkv), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
+                           eps, pos, cache_pos, plane_elems, q_norm, k_norm, inv_freq, q_proj, k_in, v_in, q_out,
+                           gate_out, (float *)k_tiled, (float *)v_tiled);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
+}
+
+}  // namespace mfa

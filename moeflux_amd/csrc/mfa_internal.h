@@ -106,6 +106,9 @@ struct FullLayer {
     void *k = nullptr;  // [Hkv] planes, tiled (see KvTile)
     void *v = nullptr;
     int32_t len = 0;
+    uint16_t *q_norm = nullptr;  // [head_dim] bf16, per-head RMS norm weights of q and k
+    uint16_t *k_norm = nullptr;
+    bool norms_set = false;
 };
 
 struct LinearLayer {
@@ -126,6 +129,10 @@ struct Ctx {
     std::vector<LinearLayer> lin;
     std::vector<void *> slabs;  // device allocations behind full[] and lin[] (layer-major)
     int32_t sweep_per_layer = 0; // 1: the token sweep launches layer by layer
+    // rotation of q and k ahead of the attention core: 1 / theta^(2i/rotary_dim) on the device
+    float *inv_freq = nullptr;
+    int32_t rotary_dim = 0;
+    float *qg_stage = nullptr;   // q and gate of mfa_full_attn_step, 2 * q_dim floats
     int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
     size_t plane_elems = 0;     // elements of one (layer, K|V, kv head) plane
     // split-K workspace
@@ -179,6 +186,11 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
                 int forced_splits, int partial_only = 0);
+// attn_prologue.hip: q/gate split, per-head norms, rotation, cache append of one token.
+int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
+                         int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,
+                         const uint16_t *k_norm, const float *inv_freq, const float *q_proj, const float *k_in,
+                         const float *v_in, float *q_out, float *gate_out, void *k_tiled, void *v_tiled);
 // sdpa_prefill.hip: the same contract for a chunk whose rows fill the machine without
 // splitting the cache (no workspace, one launch).
 bool sdpa_prefill_applies(int kv_dtype, int Hq, int Hkv, int n_tok, int64_t kv_len, int num_cus);

@@ -152,6 +152,31 @@ class Ctx:
         _chk(self.lib.mfa_sdpa_decode(self.h, layer, _p(q), _p(g), _p(out)), "mfa_sdpa_decode")
         return out
 
+    def set_full_weights(self, layer, q_norm_bf16, k_norm_bf16):
+        qn = _u16(q_norm_bf16, self.cfg.head_dim, "q_norm weight")
+        kn = _u16(k_norm_bf16, self.cfg.head_dim, "k_norm weight")
+        _chk(self.lib.mfa_set_full_weights(self.h, layer, _p(qn), _p(kn)), "mfa_set_full_weights")
+
+    def set_rope(self, theta: float, rotary_dim: int):
+        _chk(self.lib.mfa_set_rope(self.h, theta, rotary_dim), "mfa_set_rope")
+
+    def attn_prologue(self, layer, pos, q_proj_out, k, v):
+        """(q, q_gate) for the attention core; the token's k (normed, rotated) and v are appended."""
+        cfg = self.cfg
+        qp = _f32(q_proj_out, 2 * cfg.q_dim, "q_proj_out")
+        k, v = _f32(k, cfg.kv_dim, "k"), _f32(v, cfg.kv_dim, "v")
+        q, g = np.empty(cfg.q_dim, np.float32), np.empty(cfg.q_dim, np.float32)
+        _chk(self.lib.mfa_attn_prologue(self.h, layer, pos, _p(qp), _p(k), _p(v), _p(q), _p(g)), "mfa_attn_prologue")
+        return q, g
+
+    def full_attn_step(self, layer, pos, q_proj_out, k, v) -> np.ndarray:
+        cfg = self.cfg
+        qp = _f32(q_proj_out, 2 * cfg.q_dim, "q_proj_out")
+        k, v = _f32(k, cfg.kv_dim, "k"), _f32(v, cfg.kv_dim, "v")
+        out = np.empty(cfg.q_dim, np.float32)
+        _chk(self.lib.mfa_full_attn_step(self.h, layer, pos, _p(qp), _p(k), _p(v), _p(out)), "mfa_full_attn_step")
+        return out
+
     def prefill_attn(self, layer, q, q_gate, k, v) -> np.ndarray:
         q = _f32(q)
         T = q.size // self.cfg.q_dim

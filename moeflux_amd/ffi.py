@@ -48,6 +48,12 @@ SIGNATURES = {
     "mfa_gdn_step_dev": (C.c_int, [vp, i32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_prefill_gdn": (C.c_int, [vp, i32, i32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_prefill_gdn_dev": (C.c_int, [vp, i32, i32, f32p, f32p, f32p, f32p, f32p]),
+    "mfa_set_full_weights": (C.c_int, [vp, C.c_int32, u16p, u16p]),
+    "mfa_set_rope": (C.c_int, [vp, C.c_float, C.c_int32]),
+    "mfa_attn_prologue": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p, f32p]),
+    "mfa_attn_prologue_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p, f32p]),
+    "mfa_full_attn_step": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
+    "mfa_full_attn_step_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_set_sweep_per_layer": (C.c_int, [vp, C.c_int32]),
     "mfa_token_sweep_dev": (C.c_int, [vp, f32p, f32p, f32p, f32p, f32p, f32p, f32p, f32p]),
     "mfa_reset": (C.c_int, [vp]),

@@ -244,3 +244,43 @@ def prefill_gdn(T, k_heads, v_heads, key_dim, value_dim, kernel_size, eps, conv_
                                _p(alpha), _p(beta), _p(cs), _p(ss), _p(out))
     _check(rc, "orc_prefill_gdn")
     return out.reshape(T, v_heads * value_dim), cs, ss
+
+
+def rms_norm_per_head(num_heads, head_dim, eps, weight_bf16, x):
+    x = _f32(x).copy()
+    rc = lib().orc_rms_norm_per_head(C.c_int32(num_heads), C.c_int32(head_dim), C.c_float(eps),
+                                     _p(_u16(weight_bf16)), _p(x))
+    _check(rc, "orc_rms_norm_per_head")
+    return x
+
+
+def rope_inv_freq(theta, rotary_dim):
+    out = np.empty(rotary_dim // 2, dtype=np.float32)
+    _check(lib().orc_rope_inv_freq(C.c_float(theta), C.c_int32(rotary_dim), _p(out)), "orc_rope_inv_freq")
+    return out
+
+
+def apply_rotary_emb(pos, num_heads, num_kv_heads, head_dim, rotary_dim, theta, q, k):
+    """Returns (q, k) rotated at position pos."""
+    q, k = _f32(q).copy(), _f32(k).copy()
+    rc = lib().orc_apply_rotary_emb(C.c_int32(pos), C.c_int32(num_heads), C.c_int32(num_kv_heads),
+                                    C.c_int32(head_dim), C.c_int32(rotary_dim), C.c_float(theta),
+                                    _p(q), _p(k))
+    _check(rc, "orc_apply_rotary_emb")
+    return q, k
+
+
+def attn_prologue(pos, num_heads, num_kv_heads, head_dim, rotary_dim, theta, eps, q_norm_bf16,
+                  k_norm_bf16, q_proj_out, k_in, v_in):
+    """Returns (q, q_gate, k_row, v_row): the attention core's inputs and the row appended to the cache."""
+    q_proj_out, k_in, v_in = map(_f32, (q_proj_out, k_in, v_in))
+    qd, kd = num_heads * head_dim, num_kv_heads * head_dim
+    q, g = np.empty(qd, np.float32), np.empty(qd, np.float32)
+    kr, vr = np.empty(kd, np.float32), np.empty(kd, np.float32)
+    rc = lib().orc_attn_prologue(C.c_int32(pos), C.c_int32(num_heads), C.c_int32(num_kv_heads),
+                                 C.c_int32(head_dim), C.c_int32(rotary_dim), C.c_float(theta),
+                                 C.c_float(eps), _p(_u16(q_norm_bf16)), _p(_u16(k_norm_bf16)),
+                                 _p(q_proj_out), _p(k_in), _p(v_in), _p(q), _p(g), _p(kr), _p(vr))
+    _check(rc, "orc_attn_prologue")
+    return q, g, kr, vr
+

@@ -144,3 +144,26 @@ def prefill_attn(T, kv_len0, Hq, Hkv, d, q, gate, K, V):
     w = softmax(s, axis=2)
     o = np.einsum("thl,lhd->thd", w, Vx)
     return (o * expit(gate)).reshape(-1)
+
+
+def rms_norm_per_head(H, d, eps, w_bf16, x):
+    x = np.asarray(x, np.float64).reshape(H, d)
+    return (x / np.sqrt((x * x).mean(axis=1, keepdims=True) + eps) * bf16_bits_to_f64(w_bf16)).reshape(-1)
+
+
+def rotary(pos, H, d, rotary_dim, theta, x):
+    """The rotation as a complex product: channels (i, i + rotary_dim/2) of each head form
+    x_i + j x_{i+half}, multiplied by exp(j pos theta^(-2i/rotary_dim))."""
+    x = np.asarray(x, np.float64).reshape(H, d).copy()
+    half = rotary_dim // 2
+    zc = (x[:, :half] + 1j * x[:, half:rotary_dim]) * np.exp(1j * pos * theta ** (-2.0 * np.arange(half) / rotary_dim))
+    x[:, :half], x[:, half:rotary_dim] = zc.real, zc.imag
+    return x.reshape(-1)
+
+
+def attn_prologue(pos, Hq, Hkv, d, rotary_dim, theta, eps, q_norm_bf16, k_norm_bf16, q_proj_out, k_in, v_in):
+    qp = np.asarray(q_proj_out, np.float64).reshape(Hq, 2, d)
+    q = rotary(pos, Hq, d, rotary_dim, theta, rms_norm_per_head(Hq, d, eps, q_norm_bf16, qp[:, 0]))
+    k = rotary(pos, Hkv, d, rotary_dim, theta, rms_norm_per_head(Hkv, d, eps, k_norm_bf16, k_in))
+    return q, qp[:, 1].reshape(-1).copy(), k, np.asarray(v_in, np.float64).copy()
+

@@ -19,7 +19,8 @@
  *   orc_attn_values, orc_sigmoid_gate, orc_conv1d_step, orc_conv_state_shift,
  *   orc_rms_norm_bare, orc_rms_norm_qk, orc_rms_norm_gated, orc_decay_beta,
  *   orc_gated_delta_recurrence, orc_gdn_step, orc_prefill_attn,
- *   orc_prefill_gdn : pinned by float64 brute force on small shapes, closed
+ *   orc_prefill_gdn, orc_rms_norm_per_head, orc_apply_rotary_emb,
+ *   orc_attn_prologue : pinned by float64 brute force on small shapes, closed
  *   forms and invariants (the reference holds no numeric vectors for them).
  *   The Accelerate-BLAS variant of the recurrence (infer.m:4954-4993) is not
  *   restated: parity unpinned at that boundary (mathematically identical to
@@ -459,4 +460,85 @@ ORC_API int orc_prefill_gdn(int32_t T, int32_t k_heads, int32_t v_heads, int32_t
         if (rc) return rc;
     }
     return 0;
+}
+
+/* ---- what precedes the attention core in a full-attention layer -------------- */
+
+/* crates/moeflux/src/riir/rms_norm.rs:104-156 (rms_norm_per_head_cpu): each
+ * head's head_dim-long slice is normalised on its own and scaled by one shared
+ * bf16 weight vector; x * inv_rms * weight, in that order. */
+ORC_API int orc_rms_norm_per_head(int32_t num_heads, int32_t head_dim, float eps,
+                                  const uint16_t *weight_bf16, float *x_inout) {
+    if (num_heads <= 0 || head_dim <= 0 || !weight_bf16 || !x_inout) return -1;
+    const float head_dim_f = (float)head_dim;
+    for (int h = 0; h < num_heads; h++) {
+        float *xh = x_inout + (int64_t)h * head_dim;
+        float sum_sq = 0.0f;
+        for (int i = 0; i < head_dim; i++) sum_sq += xh[i] * xh[i];
+        const float inv_rms = 1.0f / sqrtf(sum_sq / head_dim_f + eps);
+        for (int i = 0; i < head_dim; i++) xh[i] = xh[i] * inv_rms * orc_bf16_to_f32(weight_bf16[i]);
+    }
+    return 0;
+}
+
+/* The frequency table of crates/moeflux/src/riir/rope.rs:99-103:
+ * inv_freq[i] = 1 / powf(theta, 2 i / rotary_dim), i < rotary_dim / 2.  The
+ * library computes the same table with the host's powf when the rotation is
+ * configured, so that no second powf implementation enters the angle. */
+ORC_API int orc_rope_inv_freq(float theta, int32_t rotary_dim, float *inv_freq) {
+    if (rotary_dim <= 0 || (rotary_dim & 1) || !inv_freq) return -1;
+    const float rdim_f = (float)rotary_dim;
+    for (int i = 0; i < rotary_dim / 2; i++) inv_freq[i] = 1.0f / powf(theta, (float)(2 * i) / rdim_f);
+    return 0;
+}
+
+/* crates/moeflux/src/riir/rope.rs:65-131 (apply_rotary_emb): the first
+ * rotary_dim channels of every q and k head are rotated, channel i paired with
+ * channel i + rotary_dim/2; angle = pos * inv_freq[i]. */
+ORC_API int orc_apply_rotary_emb(int32_t pos, int32_t num_heads, int32_t num_kv_heads,
+                                 int32_t head_dim, int32_t rotary_dim, float theta, float *q,
+                                 float *k) {
+    if (pos < 0 || !q || !k || rotary_dim <= 0 || rotary_dim > head_dim || (rotary_dim & 1)) return -1;
+    const int half = rotary_dim / 2;
+    const float pos_f = (float)pos, rdim_f = (float)rotary_dim;
+    for (int pass = 0; pass < 2; pass++) {
+        float *x = pass ? k : q;
+        const int nh = pass ? num_kv_heads : num_heads;
+        for (int h = 0; h < nh; h++) {
+            float *xh = x + (int64_t)h * head_dim;
+            for (int i = 0; i < half; i++) {
+                const float freq = 1.0f / powf(theta, (float)(2 * i) / rdim_f);
+                const float angle = pos_f * freq;
+                const float cos_a = cosf(angle), sin_a = sinf(angle);
+                const float x0 = xh[i], x1 = xh[i + half];
+                xh[i] = x0 * cos_a - x1 * sin_a;
+                xh[i + half] = x0 * sin_a + x1 * cos_a;
+            }
+        }
+    }
+    return 0;
+}
+
+/* crates/moeflux/src/riir/full_attn_forward.rs:238-293: the q projection's
+ * output is [q_h | gate_h] per head with stride 2*head_dim; q and k get the
+ * per-head norm and the rotation; v is untouched.  k_row / v_row are what is
+ * appended to the cache; q / q_gate what the attention core receives. */
+ORC_API int orc_attn_prologue(int32_t pos, int32_t num_heads, int32_t num_kv_heads,
+                              int32_t head_dim, int32_t rotary_dim, float theta, float eps,
+                              const uint16_t *q_norm_bf16, const uint16_t *k_norm_bf16,
+                              const float *q_proj_out, const float *k_in, const float *v_in,
+                              float *q, float *q_gate, float *k_row, float *v_row) {
+    if (!q_proj_out || !k_in || !v_in || !q || !q_gate || !k_row || !v_row) return -1;
+    for (int h = 0; h < num_heads; h++) {
+        memcpy(q + (int64_t)h * head_dim, q_proj_out + (int64_t)h * 2 * head_dim, sizeof(float) * head_dim);
+        memcpy(q_gate + (int64_t)h * head_dim, q_proj_out + (int64_t)h * 2 * head_dim + head_dim,
+               sizeof(float) * head_dim);
+    }
+    memcpy(k_row, k_in, sizeof(float) * (size_t)num_kv_heads * head_dim);
+    memcpy(v_row, v_in, sizeof(float) * (size_t)num_kv_heads * head_dim);
+    int rc = orc_rms_norm_per_head(num_heads, head_dim, eps, q_norm_bf16, q);
+    if (rc) return rc;
+    rc = orc_rms_norm_per_head(num_kv_heads, head_dim, eps, k_norm_bf16, k_row);
+    if (rc) return rc;
+    return orc_apply_rotary_emb(pos, num_heads, num_kv_heads, head_dim, rotary_dim, theta, q, k_row);
 }

@@ -1,4 +1,4 @@
-"""Writes tests/golden/attention_f64.json: small cases of every function on the
+"""Writes tests/golden/attention_f64.json and tests/golden/attn_prologue_f64.json: small cases of every function on the
 attention path, inputs and float64 expected outputs.
 
 The expected values come from oracle/f64ref.py — vectorised float64 numpy built
@@ -29,7 +29,26 @@ def lst(a):
     return np.asarray(a).reshape(-1).tolist()
 
 
+def prologue_cases():
+    """What precedes the attention core in a full-attention layer: q/gate split, per-head
+    norms, partial rotation (small positions: the f32 frequency table is itself 6e-8 from exact)."""
+    rng = np.random.default_rng(20261126)
+    cases = []
+    for (Hq, Hkv, d, rd, theta, pos) in [(4, 2, 16, 4, 1e7, 0), (4, 2, 16, 4, 1e7, 3), (2, 1, 32, 8, 1e7, 57),
+                                         (3, 3, 16, 16, 1e4, 9), (8, 2, 64, 16, 1e7, 100)]:
+        qn = cref.f32_to_bf16(1.0 + 0.3 * rng.standard_normal(d))
+        kn = cref.f32_to_bf16(1.0 + 0.3 * rng.standard_normal(d))
+        qp, k, v = r32(rng, Hq * 2 * d), r32(rng, Hkv * d), r32(rng, Hkv * d)
+        q, g, kr, vr = f64ref.attn_prologue(pos, Hq, Hkv, d, rd, theta, 1e-6, qn, kn, qp, k, v)
+        cases.append(dict(Hq=Hq, Hkv=Hkv, d=d, rotary_dim=rd, theta=theta, pos=pos, eps=1e-6, q_norm=lst(qn),
+                          k_norm=lst(kn), q_proj_out=lst(qp), k=lst(k), v=lst(v), q_out=lst(q), gate_out=lst(g),
+                          k_row=lst(kr), v_row=lst(vr)))
+    with open(os.path.join(HERE, "attn_prologue_f64.json"), "w") as f:
+        json.dump({"attn_prologue": cases}, f)
+
+
 def main():
+    prologue_cases()
     rng = np.random.default_rng(20261125)
     cases = {"sdpa": [], "gdn_step": [], "conv1d": [], "rms_norm_qk": [], "decay_beta": [],
              "delta_net_step": [], "rms_norm_gated": [], "prefill_attn": []}

@@ -310,3 +310,69 @@ def test_gdn_rejects_what_the_reference_rejects():
                             np.zeros(48))
     with pytest.raises(ValueError):   # zero dim (linear_attn.rs:166)
         cref.rms_norm_bare(np.zeros(0, np.float32), 1e-6)
+
+
+# ---- what precedes the attention core: per-head norm, rotation, q/gate split ------------
+
+PRO = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "attn_prologue_f64.json")))
+
+
+@pytest.mark.parametrize("c", PRO["attn_prologue"], ids=lambda c: f"Hq{c['Hq']}d{c['d']}rd{c['rotary_dim']}pos{c['pos']}")
+def test_golden_attn_prologue(c):
+    q, g, kr, vr = cref.attn_prologue(c["pos"], c["Hq"], c["Hkv"], c["d"], c["rotary_dim"], c["theta"], c["eps"],
+                                      u16(c["q_norm"]), u16(c["k_norm"]), a32(c["q_proj_out"]), a32(c["k"]),
+                                      a32(c["v"]))
+    assert rel_err(q, a32(c["q_out"])) <= 1e-5 and rel_err(kr, a32(c["k_row"])) <= 1e-5
+    assert np.array_equal(g, a32(c["gate_out"])) and np.array_equal(vr, a32(c["v_row"]))
+
+
+def test_rope_position_zero_is_the_identity():
+    """rope.rs:352-383 (the reference's own unit test): cos = 1, sin = 0 leave every channel as it was."""
+    Hq, Hkv, d = 4, 2, 32
+    q = (np.arange(Hq * d) * 0.001).astype(np.float32)
+    k = (np.arange(Hkv * d) * 0.001).astype(np.float32)
+    q2, k2 = cref.apply_rotary_emb(0, Hq, Hkv, d, d // 4, 1e7, q, k)
+    assert np.array_equal(q, q2) and np.array_equal(k, k2)
+
+
+def test_rope_is_a_rotation_of_the_paired_channels_only():
+    """Pairs (i, i + half) keep their norm, channels past rotary_dim are untouched, channel 0's
+    pair turns by exactly pos radians (theta^0 = 1), and two rotations compose: R(a) R(b) = R(a+b)
+    on the first pair, which a wrong sign in either output line breaks."""
+    rng = np.random.default_rng(3)
+    H, d, rd = 3, 32, 8
+    half = rd // 2
+    x = rng.standard_normal(H * d).astype(np.float32)
+    y, _ = cref.apply_rotary_emb(7, H, 1, d, rd, 1e7, x, x[:d])
+    X, Y = x.reshape(H, d), y.reshape(H, d)
+    assert np.array_equal(X[:, rd:], Y[:, rd:])
+    assert np.allclose(X[:, :half] ** 2 + X[:, half:rd] ** 2, Y[:, :half] ** 2 + Y[:, half:rd] ** 2, rtol=1e-5)
+    ang = np.arctan2(Y[:, half], Y[:, 0]) - np.arctan2(X[:, half], X[:, 0])
+    assert np.allclose(np.mod(ang - 7.0 + np.pi, 2 * np.pi) - np.pi, 0.0, atol=1e-5)
+    y2, _ = cref.apply_rotary_emb(5, H, 1, d, rd, 1e7, y, y[:d])
+    y12, _ = cref.apply_rotary_emb(12, H, 1, d, rd, 1e7, x, x[:d])
+    assert np.allclose(y2.reshape(H, d)[:, [0, half]], y12.reshape(H, d)[:, [0, half]], atol=2e-6)
+
+
+def test_rope_frequency_table():
+    f = cref.rope_inv_freq(1e7, 64)
+    assert f[0] == 1.0 and np.all(np.diff(f) < 0)
+    assert np.allclose(f, 1e7 ** (-2.0 * np.arange(32) / 64), rtol=3e-7)
+
+
+def test_rms_norm_per_head_properties():
+    """Unit weight: every head leaves with mean square 1; a head's scale does not leak into
+    another head; scaling the input leaves the output unchanged (up to eps)."""
+    rng = np.random.default_rng(4)
+    H, d = 5, 64
+    one = cref.f32_to_bf16(np.ones(d))
+    x = rng.standard_normal(H * d).astype(np.float32)
+    y = cref.rms_norm_per_head(H, d, 1e-6, one, x).reshape(H, d)
+    assert np.allclose((y.astype(np.float64) ** 2).mean(axis=1), 1.0, rtol=1e-5)
+    x2 = x.copy().reshape(H, d)
+    x2[2] *= 37.0
+    y2 = cref.rms_norm_per_head(H, d, 1e-6, one, x2).reshape(H, d)
+    assert np.array_equal(np.delete(y, 2, axis=0), np.delete(y2, 2, axis=0)) and rel_err(y2[2], y[2]) <= 1e-6
+    w = cref.f32_to_bf16(1.0 + 0.2 * rng.standard_normal(d))
+    yw = cref.rms_norm_per_head(H, d, 1e-6, w, x).reshape(H, d)
+    assert rel_err(yw, y * cref.bf16_to_f32(w)) <= 1e-6
