@@ -239,6 +239,19 @@ int mfa_linear_state_export(mfa_ctx *ctx, int32_t layer, float *conv_state_out,
 int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state,
                             const float *ssm_state);
 
+/* The whole context's state in the reference's snapshot wire format ('MFLX',
+ * state_snapshot.rs:1-73; state_size :184-216, state_save :218-360, state_load
+ * :362-640): header of 10 little-endian u32, then per layer `i32 len` + K rows + V
+ * rows ([len, num_kv_heads*head_dim] f32) or conv state + recurrent state.  Saved
+ * as version 2 with both MLA fields 0; versions 1 and 2 load.  Call at token
+ * boundaries only (moeflux.h:614-617).  mfa_state_size / mfa_state_save return a
+ * byte count or a negative code; mfa_state_load checks the whole buffer before
+ * it restores anything (MFA_ERR_STATE for magic, version, shape, truncation,
+ * negative length; MFA_ERR_OVERFLOW for a length beyond kv_capacity). */
+int64_t mfa_state_size(mfa_ctx *ctx);
+int64_t mfa_state_save(mfa_ctx *ctx, uint8_t *buf, int64_t buf_len);
+int mfa_state_load(mfa_ctx *ctx, const uint8_t *buf, int64_t buf_len);
+
 /* ---- timing ---------------------------------------------------------------- */
 
 /* hipEvent pair on the context's stream (the reference's counterpart is the

@@ -250,6 +250,24 @@ class Ctx:
         _chk(self.lib.mfa_linear_state_import(self.h, layer, _p(conv), _p(ssm)),
              "mfa_linear_state_import")
 
+    def state_size(self) -> int:
+        n = self.lib.mfa_state_size(self.h)
+        if n < 0:
+            _chk(int(n), "mfa_state_size")
+        return int(n)
+
+    def state_save(self) -> bytes:
+        """The snapshot in the reference's 'MFLX' wire format (state_snapshot.rs)."""
+        buf = np.empty(self.state_size(), dtype=np.uint8)
+        n = self.lib.mfa_state_save(self.h, _p(buf), buf.size)
+        if n < 0:
+            _chk(int(n), "mfa_state_save")
+        return buf[:int(n)].tobytes()
+
+    def state_load(self, blob: bytes):
+        buf = np.frombuffer(blob, dtype=np.uint8)
+        _chk(self.lib.mfa_state_load(self.h, _p(buf) if buf.size else None, buf.size), "mfa_state_load")
+
     def sync(self):
         _chk(self.lib.mfa_sync(self.h), "mfa_sync")
 

@@ -54,6 +54,9 @@ SIGNATURES = {
     "mfa_attn_prologue_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
+    "mfa_state_size": (C.c_int64, [vp]),
+    "mfa_state_save": (C.c_int64, [vp, vp, C.c_int64]),
+    "mfa_state_load": (C.c_int, [vp, vp, C.c_int64]),
     "mfa_set_sweep_per_layer": (C.c_int, [vp, C.c_int32]),
     "mfa_token_sweep_dev": (C.c_int, [vp, f32p, f32p, f32p, f32p, f32p, f32p, f32p, f32p]),
     "mfa_reset": (C.c_int, [vp]),
