@@ -309,6 +309,74 @@ def cpu_baseline(sample, Hq, Hkv, d, L, budget_s=12.0):
                       f"(kv_len {L}, f32-widened cache), single thread"}, err
 
 
+def cpu_baseline_all_cores(sample, Hq, Hkv, d, L):
+    """The same oracle function with the query heads spread over the host cores this process
+    may use (heads are independent; the reference's own CPU path is single-threaded)."""
+    import os
+    from concurrent.futures import ThreadPoolExecutor
+    from oracle import cref
+    q, g, k, v, _ = sample
+    kf = (cref.bf16_to_f32(k) if k.dtype == np.uint16 else k).reshape(L, Hkv, d)
+    vf = (cref.bf16_to_f32(v) if v.dtype == np.uint16 else v).reshape(L, Hkv, d)
+    cores = max(1, min(len(os.sched_getaffinity(0)), 16, Hq))
+    kh = [np.ascontiguousarray(kf[:, h]) for h in range(Hkv)]
+    vh = [np.ascontiguousarray(vf[:, h]) for h in range(Hkv)]
+    hpk = Hq // Hkv
+    qs, gs = q.reshape(Hq, d), g.reshape(Hq, d)
+
+    def one(h):  # ctypes drops the GIL for the duration of the call
+        return cref.sdpa(L, 1, 1, d, qs[h], gs[h], kh[h // hpk], vh[h // hpk])
+
+    with ThreadPoolExecutor(cores) as ex:
+        list(ex.map(one, range(Hq)))
+        t0 = time.perf_counter()
+        n = 3
+        for _ in range(n):
+            list(ex.map(one, range(Hq)))
+        per = (time.perf_counter() - t0) / n
+    return {"value": per * 1e6, "unit": "us/layer/token", "cores": cores, "kind": "port",
+            "sample": f"{n} calls, the {Hq} query heads of orc_sdpa spread over {cores} threads"}
+
+
+def cpu_secondary():
+    """One-thread oracle timings of the secondary configurations, same shapes, bounded samples."""
+    from oracle import cref
+    from tests.util import GdnCase
+    rng = np.random.default_rng(1)
+
+    def timed(fn, n):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    def sdpa_inputs(Hq, Hkv, d, L):
+        return (rng.standard_normal(Hq * d, dtype=np.float32), rng.standard_normal(Hq * d, dtype=np.float32),
+                rng.standard_normal((L, Hkv * d), dtype=np.float32), rng.standard_normal((L, Hkv * d), dtype=np.float32))
+
+    out = {}
+    q, g, k, v = sdpa_inputs(32, 4, 128, 4096)
+    out["c1_us_per_layer_token"] = timed(lambda: cref.sdpa(4096, 32, 4, 128, q, g, k, v), 5)
+    c = GdnCase(2, 16, 32, 128, 128, T=1, plain=True)
+    step = lambda: cref.gdn_step(16, 32, 128, 128, 4, 1e-6, c.conv_w, c.a_log, c.dt_bias, c.norm_w, c.qkv[0],
+                                 c.z[0], c.alpha[0], c.beta[0], c.conv_state, c.ssm_state)
+    out["c2_us_per_layer_token"] = timed(step, 20)
+    T = 512
+    qq = rng.standard_normal((T, 32 * 128), dtype=np.float32)
+    kk = rng.standard_normal((T, 4 * 128), dtype=np.float32)
+    out["c4_attention_us_per_chunk"] = timed(lambda: cref.prefill_attn(T, 0, 32, 4, 128, qq, qq, kk, kk), 1)
+    out["c4_deltanet_us_per_chunk"] = out["c2_us_per_layer_token"] * T
+    q, g, k, v = sdpa_inputs(32, 2, 256, 8192)
+    full = timed(lambda: cref.sdpa(8192, 32, 2, 256, q, g, k, v), 3)
+    out["c5_us_per_token_sweep"] = 36 * out["c2_us_per_layer_token"] + 12 * full
+    out["cores"] = 1
+    out["kind"] = "port"
+    out["sample"] = ("oracle functions at the full shapes: c1 5 calls, c2 20 calls, c4 attention one 512-token "
+                     "chunk, c4 DeltaNet = 512 x the c2 step, c5 = 36 x the c2 step + 12 x orc_sdpa at kv_len 8192 (3 calls)")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -357,6 +425,7 @@ def main():
     }
     if not a.no_cpu:
         line["cpu_baseline"], line["gpu_vs_oracle_rel_err"] = cpu_baseline(sample, Hq, Hkv, d, L)
+        line["cpu_baseline_all_cores"] = cpu_baseline_all_cores(sample, Hq, Hkv, d, L)
     else:
         line["cpu_baseline"] = None
     del sample
@@ -368,6 +437,8 @@ def main():
                                                     0xC0FFEE + 2)
         extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
         extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
+        if not a.no_cpu:
+            extra["cpu_one_thread"] = cpu_secondary()
         line["extra"] = extra
     print(json.dumps(line))
 
