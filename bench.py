@@ -309,6 +309,54 @@ def cpu_baseline(sample, Hq, Hkv, d, L, budget_s=12.0):
                       f"(kv_len {L}, f32-widened cache), single thread"}, err
 
 
+def bench_matvec(steps, warmup, seed):
+    """The projections either side of the attention core at the A17B variant's shapes
+    (variants.rs:384-400): q, k and v projections of a full-attention layer in one launch
+    ([16384 + 512 + 512, 4096] 4-bit group-64 weights) and o_proj ([4096, 8192]); weight sets
+    rotated so that every launch reads its weights from HBM."""
+    import ctypes as C
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    lib = ffi.load()
+    ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64, kv_capacity=4))
+    rng = np.random.default_rng(seed)
+    res, keep = {}, []
+
+    def weights(od, idim):
+        w = DeviceArray.from_host(rng.integers(0, 2 ** 32, size=(od, idim // 8), dtype=np.uint64).astype(np.uint32))
+        sc = DeviceArray.from_host(np.full((od, idim // 64), 0x3C00, np.uint16))
+        bi = DeviceArray.from_host(np.full((od, idim // 64), 0xBD00, np.uint16))
+        keep.extend([w, sc, bi])
+        return w, sc, bi
+
+    for name, shapes, idim, nsets in (("qkv_proj", (16384, 512, 512), 4096, 8), ("o_proj", (4096,), 8192, 14)):
+        x = DeviceArray.from_host(rng.standard_normal(idim).astype(np.float32))
+        keep.append(x)
+        sets = []
+        for _ in range(nsets):
+            specs = (ffi.mfa_matvec_spec * len(shapes))()
+            for i, od in enumerate(shapes):
+                w, sc, bi = weights(od, idim)
+                o = DeviceArray((od,), np.float32, zero=True)
+                keep.append(o)
+                specs[i] = ffi.mfa_matvec_spec(w.ptr, sc.ptr, bi.ptr, x.ptr, o.ptr, od, idim)
+            sets.append(specs)
+
+        def step(i, sets=sets, n=len(shapes)):
+            if lib.mfa_dequant_matvec_4bit_dev(ctx.h, n, C.byref(sets[i % len(sets)])) != 0:
+                raise RuntimeError(ffi.last_error())
+
+        wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
+        nw = sum(shapes) * idim
+        alg = nw // 2 + (nw // 64) * 4 + idim * 4 + sum(shapes) * 4
+        res[name] = {"shapes": [[od, idim] for od in shapes], "us_per_launch": ev_ms * 1e3, "algorithmic_bytes": alg,
+                     "gbps": alg / (ev_ms * 1e-3) / 1e9, "pct_peak": 100.0 * alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    ctx.close()
+    for a in keep:
+        a.free()
+    return res
+
+
 def cpu_baseline_all_cores(sample, Hq, Hkv, d, L):
     """The same oracle function with the query heads spread over the host cores this process
     may use (heads are independent; the reference's own CPU path is single-threaded)."""
@@ -387,7 +435,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
-    ap.add_argument("--only", choices=["c4", "c5"], default=None,
+    ap.add_argument("--only", choices=["c4", "c5", "f3"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -400,6 +448,9 @@ def main():
 
     if a.only == "c4":
         print(json.dumps({"c4_prefill_chunk_512": bench_prefill(a.steps, a.warmup, 0xC0FFEE + 4)}))
+        return
+    if a.only == "f3":
+        print(json.dumps({"f3_projection_matvecs": bench_matvec(a.steps, a.warmup, 0xC0FFEE + 6)}))
         return
     if a.only == "c5":
         print(json.dumps({"c5_token_sweep_48_layers": bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)}))
@@ -437,6 +488,7 @@ def main():
                                                     0xC0FFEE + 2)
         extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
         extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
+        extra["f3_projection_matvecs"] = bench_matvec(a.steps // 2, a.warmup, 0xC0FFEE + 6)
         if not a.no_cpu:
             extra["cpu_one_thread"] = cpu_secondary()
         line["extra"] = extra

@@ -123,6 +123,33 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
 int mfa_sdpa_decode_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev,
                         const float *q_gate_dev, float *out_dev);
 
+/* ---- the projections either side of the attention core ------------------------ */
+
+/* One 4-bit group-64 affine dequantising matrix-vector product, all pointers on
+ * the device: w_packed [out_dim, in_dim/8] u32 (nibble n of a word is input
+ * 8*word+n), scales, biases [out_dim, in_dim/64] bf16, x [in_dim], out [out_dim]. */
+typedef struct mfa_matvec_spec {
+    const uint32_t *w_packed;
+    const uint16_t *scales;
+    const uint16_t *biases;
+    const float *x;
+    float *out;
+    int32_t out_dim;
+    int32_t in_dim;
+} mfa_matvec_spec;
+
+/* Replaces the batched dequant_matvec_4bit_v3 dispatches that feed and drain the
+ * attention core (shaders.metal:251-340; encoders gpu_matvec.rs; call sites
+ * full_attn_forward.rs:193-227 for q/k/v_proj, linear_attn_forward.rs:560-605 for
+ * in_proj_qkv/z/a/b, and o_proj / out_proj): n (1..8) products in one launch on
+ * the context's stream.  in_dim a multiple of 64, at most 8192. */
+int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs);
+/* Stateless host-pointer twin of dequant_matvec_4bit_cpu (cpu_matvec.rs:83-160;
+ * cpu_dequant_matvec, infer.m:671).  group_size must be 64. */
+int mfa_dequant_matvec_4bit(int32_t out_dim, int32_t in_dim, int32_t group_size,
+                            const uint32_t *w_packed, const uint16_t *scales,
+                            const uint16_t *biases, const float *x, float *out);
+
 /* ---- what precedes the attention core in a full-attention layer -------------- */
 
 /* Per-layer constants of the prologue: the bf16 weights of the per-head RMS

@@ -763,6 +763,45 @@ int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on) {
     return MFA_OK;
 }
 
+/* ---- projections ------------------------------------------------------------------- */
+
+int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs) {
+    Ctx *c = as_ctx(ctx);
+    if (!c || !specs) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (n <= 0 || n > 8) return fail(MFA_ERR_INVALID, "1 to 8 products per call (got %d)", n);
+    const uint32_t *w[8];
+    const uint16_t *sc[8], *bi[8];
+    const float *x[8];
+    float *out[8];
+    int od[8], id[8];
+    for (int i = 0; i < n; i++) {
+        w[i] = specs[i].w_packed; sc[i] = specs[i].scales; bi[i] = specs[i].biases;
+        x[i] = specs[i].x; out[i] = specs[i].out; od[i] = specs[i].out_dim; id[i] = specs[i].in_dim;
+    }
+    return launch_dequant_matvec_4bit(c->stream, n, w, sc, bi, x, out, od, id, c->num_cus);
+}
+
+int mfa_dequant_matvec_4bit(int32_t out_dim, int32_t in_dim, int32_t group_size, const uint32_t *w_packed,
+                            const uint16_t *scales, const uint16_t *biases, const float *x, float *out) {
+    if (!w_packed || !scales || !biases || !x || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (out_dim <= 0 || in_dim <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (group_size != 64) return fail(MFA_ERR_SHAPE, "group size %d not supported (64)", group_size);
+    if (in_dim % 64 != 0) return fail(MFA_ERR_INVALID, "in_dim %d is not a multiple of the group size 64", in_dim);
+    const size_t nw = (size_t)out_dim * (in_dim / 8), ng = (size_t)out_dim * (in_dim / 64);
+    DevBuf dw, ds, db, dx, dout;
+    MFA_TRY(dw.upload(w_packed, nw * 4));
+    MFA_TRY(ds.upload(scales, ng * 2));
+    MFA_TRY(db.upload(biases, ng * 2));
+    MFA_TRY(dx.upload(x, (size_t)in_dim * 4));
+    MFA_TRY(dout.alloc((size_t)out_dim * 4));
+    const uint32_t *w[1] = {dw.as<uint32_t>()};
+    const uint16_t *sc[1] = {ds.as<uint16_t>()}, *bi[1] = {db.as<uint16_t>()};
+    const float *xx[1] = {dx.as<float>()};
+    float *oo[1] = {dout.as<float>()};
+    MFA_TRY(launch_dequant_matvec_4bit(nullptr, 1, w, sc, bi, xx, oo, &out_dim, &in_dim));
+    return dout.download(out, (size_t)out_dim * 4);
+}
+
 /* ---- state operations ----------------------------------------------------------- */
 
 int mfa_reset(mfa_ctx *ctx) {

@@ -186,6 +186,10 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
                 int forced_splits, int partial_only = 0);
+// dequant_matvec.hip: up to 8 four-bit dequantising matrix-vector products in one launch.
+int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const *w, const uint16_t *const *scales,
+                               const uint16_t *const *biases, const float *const *x, float *const *out,
+                               const int *out_dim, const int *in_dim, int num_cus = 256);
 // attn_prologue.hip: q/gate split, per-head norms, rotation, cache append of one token.
 int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
                          int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,

@@ -407,3 +407,18 @@ def rms_norm_gated_cpu(x, z, weight_bf16, eps):
     """`RsCtx::rms_norm_gated_cpu` (riir/mod.rs:526): the one-head case."""
     x = _f32(x)
     return gated_rms_norm(1, x.size, eps, x, z, weight_bf16)
+
+
+def dequant_matvec_4bit_cpu(packed, scales_bf16, biases_bf16, in_dim, out_dim, x):
+    """The reference hook of the same name (cpu_matvec.rs:83-160), computed on the GPU."""
+    lib = ffi.load()
+    packed = np.ascontiguousarray(packed, dtype=np.uint32).reshape(-1)
+    if packed.size != out_dim * (in_dim // 8):
+        raise ValueError(f"packed has {packed.size} words, expected {out_dim * (in_dim // 8)}")
+    sc = _u16(scales_bf16, out_dim * (in_dim // 64), "scales")
+    bi = _u16(biases_bf16, out_dim * (in_dim // 64), "biases")
+    x = _f32(x, in_dim, "x")
+    out = np.empty(out_dim, dtype=np.float32)
+    _chk(lib.mfa_dequant_matvec_4bit(out_dim, in_dim, 64, _p(packed), _p(sc), _p(bi), _p(x), _p(out)),
+         "mfa_dequant_matvec_4bit")
+    return out

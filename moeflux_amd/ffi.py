@@ -18,6 +18,11 @@ KV_F32, KV_BF16 = 0, 1
 i32, f32, vp, u16p, f32p = C.c_int32, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p
 
 
+class mfa_matvec_spec(C.Structure):
+    _fields_ = [("w_packed", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p), ("x", C.c_void_p),
+                ("out", C.c_void_p), ("out_dim", C.c_int32), ("in_dim", C.c_int32)]
+
+
 class mfa_config(C.Structure):
     _fields_ = [
         ("num_layers", i32), ("full_attn_interval", i32), ("num_attn_heads", i32),
@@ -54,6 +59,8 @@ SIGNATURES = {
     "mfa_attn_prologue_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
+    "mfa_dequant_matvec_4bit_dev": (C.c_int, [vp, C.c_int32, vp]),
+    "mfa_dequant_matvec_4bit": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, vp, u16p, u16p, f32p, f32p]),
     "mfa_state_size": (C.c_int64, [vp]),
     "mfa_state_save": (C.c_int64, [vp, vp, C.c_int64]),
     "mfa_state_load": (C.c_int, [vp, vp, C.c_int64]),

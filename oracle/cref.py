@@ -284,3 +284,12 @@ def attn_prologue(pos, num_heads, num_kv_heads, head_dim, rotary_dim, theta, eps
     _check(rc, "orc_attn_prologue")
     return q, g, kr, vr
 
+
+def dequant_matvec_4bit(packed, scales_bf16, biases_bf16, in_dim, out_dim, x):
+    packed = np.ascontiguousarray(packed, dtype=np.uint32)
+    out = np.empty(out_dim, dtype=np.float32)
+    rc = lib().orc_dequant_matvec_4bit(_p(packed), _p(_u16(scales_bf16)), _p(_u16(biases_bf16)),
+                                       C.c_int32(in_dim), C.c_int32(out_dim), _p(_f32(x)), _p(out))
+    _check(rc, "orc_dequant_matvec_4bit")
+    return out
+

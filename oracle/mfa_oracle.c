@@ -20,7 +20,7 @@
  *   orc_rms_norm_bare, orc_rms_norm_qk, orc_rms_norm_gated, orc_decay_beta,
  *   orc_gated_delta_recurrence, orc_gdn_step, orc_prefill_attn,
  *   orc_prefill_gdn, orc_rms_norm_per_head, orc_apply_rotary_emb,
- *   orc_attn_prologue : pinned by float64 brute force on small shapes, closed
+ *   orc_attn_prologue, orc_dequant_matvec_4bit : pinned by float64 brute force on small shapes, closed
  *   forms and invariants (the reference holds no numeric vectors for them).
  *   The Accelerate-BLAS variant of the recurrence (infer.m:4954-4993) is not
  *   restated: parity unpinned at that boundary (mathematically identical to
@@ -541,4 +541,36 @@ ORC_API int orc_attn_prologue(int32_t pos, int32_t num_heads, int32_t num_kv_hea
     rc = orc_rms_norm_per_head(num_kv_heads, head_dim, eps, k_norm_bf16, k_row);
     if (rc) return rc;
     return orc_apply_rotary_emb(pos, num_heads, num_kv_heads, head_dim, rotary_dim, theta, q, k_row);
+}
+
+/* ---- the projections either side of the attention core ------------------------ */
+
+/* crates/moeflux/src/riir/cpu_matvec.rs:83-160 (dequant_matvec_4bit_cpu; C twin
+ * cpu_dequant_matvec, infer.m:671): out[r] = sum_c (nibble(r,c) * scale + bias) * x[c],
+ * weights packed 8 nibbles per u32 (nibble n of a word at bits 4n..4n+3), one bf16
+ * scale and one bf16 bias per group of 64 inputs; both steps are mul_add. */
+ORC_API int orc_dequant_matvec_4bit(const uint32_t *packed, const uint16_t *scales,
+                                    const uint16_t *biases, int32_t in_dim, int32_t out_dim,
+                                    const float *x, float *out) {
+    if (!packed || !scales || !biases || !x || !out || in_dim <= 0 || out_dim <= 0) return -1;
+    if (in_dim % 64 != 0) return -1;
+    const int in_packed = in_dim / 8, in_groups = in_dim / 64;
+    for (int r = 0; r < out_dim; r++) {
+        const uint32_t *row = packed + (int64_t)r * in_packed;
+        float acc = 0.0f;
+        for (int g = 0; g < in_groups; g++) {
+            const float scale = orc_bf16_to_f32(scales[(int64_t)r * in_groups + g]);
+            const float bias = orc_bf16_to_f32(biases[(int64_t)r * in_groups + g]);
+            for (int p = 0; p < 8; p++) {
+                const uint32_t word = row[g * 8 + p];
+                for (int n = 0; n < 8; n++) {
+                    const float nibble = (float)((word >> (n * 4)) & 0xFu);
+                    const float w = fmaf(nibble, scale, bias);
+                    acc = fmaf(w, x[g * 64 + p * 8 + n], acc);
+                }
+            }
+        }
+        out[r] = acc;
+    }
+    return 0;
 }

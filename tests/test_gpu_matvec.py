@@ -1,0 +1,84 @@
+"""GPU parity of the 4-bit dequantising matrix-vector product (the projections either side
+of the attention core) against the CPU oracle, through the C ABI."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from tests.util import TOL_F32, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _weights(rng, out_dim, in_dim, oracle):
+    packed = rng.integers(0, 2 ** 32, size=(out_dim, in_dim // 8), dtype=np.uint64).astype(np.uint32)
+    # MLX affine 4-bit: scale = (max - min) / 15, bias = min of a group of 64 weights
+    sc = oracle.f32_to_bf16(np.abs(rng.standard_normal((out_dim, in_dim // 64))) * 0.01 + 0.002)
+    bi = oracle.f32_to_bf16(-7.5 * oracle.bf16_to_f32(sc) + rng.standard_normal((out_dim, in_dim // 64)) * 0.003)
+    return packed, sc, bi
+
+
+def test_reference_unit_vectors(mfa):
+    """cpu_matvec.rs:366-417: the reference's known answers, bit for bit."""
+    ones = np.ones(64, np.float32)
+    f = mfa.dequant_matvec_4bit_cpu
+    assert f(np.full(8, 0x11111111, np.uint32), [0x3F80], [0x0000], 64, 1, ones)[0] == 64.0
+    assert np.array_equal(f(np.full(16, 0xFFFFFFFF, np.uint32), [0x3F80] * 2, [0x3F80] * 2, 64, 2, np.zeros(64, np.float32)),
+                          np.zeros(2, np.float32))
+    assert f(np.zeros(8, np.uint32), [0x40A0], [0x4000], 64, 1, ones)[0] == 128.0
+
+
+@pytest.mark.parametrize("out_dim,in_dim", [(1, 64), (5, 192), (33, 2048), (512, 4096), (100, 4160), (4096, 8192),
+                                            (16384, 4096), (37, 1024)])
+def test_matvec_matches_oracle(mfa, oracle, out_dim, in_dim):
+    """Projection shapes of the variants (q_proj 16384x4096, k/v_proj 512x4096, o_proj 4096x8192,
+    expert down_proj x1024) and ragged ones: row counts that do not fill a workgroup, widths that
+    do not fill the last 2048-input chunk."""
+    rng = np.random.default_rng(out_dim + in_dim)
+    packed, sc, bi = _weights(rng, out_dim, in_dim, oracle)
+    x = rng.standard_normal(in_dim).astype(np.float32)
+    ref = oracle.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, x)
+    out = mfa.dequant_matvec_4bit_cpu(packed, sc, bi, in_dim, out_dim, x)
+    assert rel_err(out, ref) <= TOL_F32
+
+
+def test_batched_products_in_one_launch(mfa, oracle):
+    """q, k and v projections of one layer as one call on device pointers
+    (full_attn_forward.rs:193-227 batches them into one command buffer)."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    rng = np.random.default_rng(4)
+    in_dim = 4096
+    x = rng.standard_normal(in_dim).astype(np.float32)
+    shapes = [16384, 512, 512]
+    dx = DeviceArray.from_host(x)
+    keep, refs, outs = [dx], [], []
+    specs = (ffi.mfa_matvec_spec * 3)()
+    for i, od in enumerate(shapes):
+        packed, sc, bi = _weights(rng, od, in_dim, oracle)
+        refs.append(oracle.dequant_matvec_4bit(packed, sc, bi, in_dim, od, x))
+        dw, ds, db = DeviceArray.from_host(packed), DeviceArray.from_host(sc), DeviceArray.from_host(bi)
+        do = DeviceArray((od,), np.float32, zero=True)
+        keep += [dw, ds, db]
+        outs.append(do)
+        specs[i] = ffi.mfa_matvec_spec(dw.ptr, ds.ptr, db.ptr, dx.ptr, do.ptr, od, in_dim)
+    with mfa.Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64,
+                        kv_capacity=4)) as c:
+        rc = c.lib.mfa_dequant_matvec_4bit_dev(c.h, 3, C.byref(specs))
+        assert rc == 0, ffi.last_error()
+        c.sync()
+        for o, r in zip(outs, refs):
+            assert rel_err(o.to_host(), r) <= TOL_F32
+
+
+def test_matvec_errors(mfa):
+    """cpu_matvec.rs:92-97: in_dim must be a multiple of the group size; NULL and shape checks."""
+    from moeflux_amd import ffi
+    lib = ffi.load()
+    w, s, x, o = np.zeros(8, np.uint32), np.zeros(1, np.uint16), np.zeros(64, np.float32), np.zeros(1, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    assert lib.mfa_dequant_matvec_4bit(1, 32, 64, p(w), p(s), p(s), p(x), p(o)) == ffi.ERR_INVALID
+    assert lib.mfa_dequant_matvec_4bit(1, 64, 32, p(w), p(s), p(s), p(x), p(o)) == ffi.ERR_SHAPE
+    assert lib.mfa_dequant_matvec_4bit(0, 64, 64, p(w), p(s), p(s), p(x), p(o)) == ffi.ERR_INVALID
+    assert lib.mfa_dequant_matvec_4bit(1, 64, 64, None, p(s), p(s), p(x), p(o)) == ffi.ERR_INVALID
+    assert lib.mfa_dequant_matvec_4bit(1, 64, 64, p(w), p(s), p(s), p(x), p(o)) == 0

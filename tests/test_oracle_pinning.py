@@ -376,3 +376,37 @@ def test_rms_norm_per_head_properties():
     w = cref.f32_to_bf16(1.0 + 0.2 * rng.standard_normal(d))
     yw = cref.rms_norm_per_head(H, d, 1e-6, w, x).reshape(H, d)
     assert rel_err(yw, y * cref.bf16_to_f32(w)) <= 1e-6
+
+
+# ---- 4-bit dequantising matvec (the projections either side of the attention core) -------
+
+def test_dequant_matvec_reference_unit_tests():
+    """cpu_matvec.rs:366-417, the reference's own known-answer tests: all nibbles 1 with
+    scale 1 bias 0 against ones gives 64; a zero input gives zero whatever the bias; nibble 0
+    with bias 2 against ones gives 128."""
+    ones = np.ones(64, np.float32)
+    assert cref.dequant_matvec_4bit(np.full(8, 0x11111111, np.uint32), [0x3F80], [0x0000], 64, 1, ones)[0] == 64.0
+    out = cref.dequant_matvec_4bit(np.full(16, 0xFFFFFFFF, np.uint32), [0x3F80] * 2, [0x3F80] * 2, 64, 2,
+                                   np.zeros(64, np.float32))
+    assert np.array_equal(out, np.zeros(2, np.float32))
+    assert cref.dequant_matvec_4bit(np.zeros(8, np.uint32), [0x40A0], [0x4000], 64, 1, ones)[0] == 128.0
+
+
+def test_dequant_matvec_against_float64_matrix_product():
+    """Unpack the nibbles with numpy (bit n*4 of each word is input 8*word + n), build the
+    dequantised matrix in float64 and multiply: pins nibble order, group stride and row stride."""
+    rng = np.random.default_rng(8)
+    out_dim, in_dim = 7, 256
+    packed = rng.integers(0, 2 ** 32, size=(out_dim, in_dim // 8), dtype=np.uint64).astype(np.uint32)
+    sc = cref.f32_to_bf16(rng.standard_normal((out_dim, in_dim // 64)) * 0.1)
+    bi = cref.f32_to_bf16(rng.standard_normal((out_dim, in_dim // 64)) * 0.5)
+    x = rng.standard_normal(in_dim).astype(np.float32)
+    nib = ((packed[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF).reshape(out_dim, in_dim).astype(np.float64)
+    W = nib * np.repeat(cref.bf16_to_f32(sc).astype(np.float64), 64, axis=1) + \
+        np.repeat(cref.bf16_to_f32(bi).astype(np.float64), 64, axis=1)
+    got = cref.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, x)
+    assert rel_err(got, (W @ x.astype(np.float64)).astype(np.float32)) <= 2e-6
+    # linear in x; a one-hot x picks one dequantised column
+    e = np.zeros(in_dim, np.float32)
+    e[77] = 1.0
+    assert np.allclose(cref.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, e), W[:, 77], rtol=1e-6)
