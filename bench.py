@@ -148,7 +148,7 @@ def bench_gdn(name, Hk, Hv, dk, dv, layers, steps, warmup, seed):
     return res
 
 
-def bench_prefill(steps, warmup, seed):
+def bench_prefill(steps, warmup, seed, T=512):
     """BASELINE configs[3]: a 512-token prompt chunk from an empty cache / zero state —
     causal GQA attention (32 Q / 4 KV heads, d=128, bf16 cache) and the Gated-DeltaNet
     chunk (configs[1] shape).  Every timed call uses a fresh layer, so kv_len0 = 0."""
@@ -156,7 +156,7 @@ def bench_prefill(steps, warmup, seed):
     from moeflux_amd.hip import DeviceArray
     from tests.util import GdnCase
     lib = ffi.load()
-    T, Hq, Hkv, d = 512, 32, 4, 128
+    Hq, Hkv, d = 32, 4, 128
     n = steps + warmup
     rng = np.random.default_rng(seed)
     ctx = Ctx(Config(num_layers=n, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
@@ -435,6 +435,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
+    ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
     ap.add_argument("--only", choices=["c4", "c5", "f3"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
@@ -447,7 +448,7 @@ def main():
         return
 
     if a.only == "c4":
-        print(json.dumps({"c4_prefill_chunk_512": bench_prefill(a.steps, a.warmup, 0xC0FFEE + 4)}))
+        print(json.dumps({f"c4_prefill_chunk_{a.tokens}": bench_prefill(a.steps, a.warmup, 0xC0FFEE + 4, a.tokens)}))
         return
     if a.only == "f3":
         print(json.dumps({"f3_projection_matvecs": bench_matvec(a.steps, a.warmup, 0xC0FFEE + 6)}))

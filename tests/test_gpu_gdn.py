@@ -153,3 +153,57 @@ def test_config4_gdn_chunk_of_512_from_zero_state(mfa):
     assert worst <= 5e-5
     assert np.array_equal(conv.reshape(-1), ref_conv)
     assert rel_err(ssm, ref_ssm) <= TOL_F32
+
+
+def _same_tokens(c):
+    c.qkv[:] = c.qkv[0]
+
+
+def _same_tokens_beta_one(c):
+    c.qkv[:] = c.qkv[0]
+    c.beta[:] = 20.0
+    c.alpha[:] = -20.0
+
+
+def _drift(c):
+    d = np.random.default_rng(1).standard_normal(c.qkv.shape).astype(np.float32) * 0.02
+    c.qkv[:] = c.qkv[0] + np.cumsum(d, axis=0)
+
+
+def _strong_decay(c):
+    c.alpha[:] = 8.0
+    c.a_log[:] = 1.5
+
+
+def _big(c):
+    c.qkv *= 30.0
+
+
+@pytest.mark.parametrize("mutate", [_same_tokens, _same_tokens_beta_one, _drift, _strong_decay, _big],
+                         ids=["identical-tokens", "identical-tokens-beta1-g1", "drifting-tokens", "strong-decay",
+                              "inputs-x30"])
+def test_blocked_form_on_hard_inputs(mfa, mutate):
+    """The blocked form inverts I + A per 64-token block, A built from key-key products: keys that
+    repeat or drift slowly make A dense with entries near beta, gates at their extremes stretch the
+    decay factors (e^{L_C} underflows under strong decay).  Same criterion as everywhere."""
+    case = GdnCase(5, 2, 4, 128, 128, T=256)
+    mutate(case)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case) as c:
+        c.linear_state_import(0, case.conv_state, case.ssm_state)
+        out = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
+        conv, ssm = c.linear_state_export(0)
+    assert np.isfinite(out).all()
+    assert rel_err(out, ref_out) <= TOL_F32 and rel_err(ssm, ref_ssm) <= TOL_F32
+    assert np.array_equal(conv.reshape(-1), ref_conv)
+
+
+def test_chunk_at_the_a17b_head_counts(mfa):
+    """16 key heads, 64 value heads (variants.rs:396-397), a ragged 130-token chunk."""
+    case = GdnCase(6, 16, 64, 128, 128, T=130)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case) as c:
+        c.linear_state_import(0, case.conv_state, case.ssm_state)
+        out = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
+        _, ssm = c.linear_state_export(0)
+    assert rel_err(out, ref_out) <= TOL_F32 and rel_err(ssm, ref_ssm) <= TOL_F32
