@@ -298,29 +298,29 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
     };
     float4 pw[NK], pq[NK], pu;
     auto slot_of = [&](int blk) { return (size_t)(blk < nblk ? blk : nblk - 1) * Hv + vh; };
-    auto fetch_wq = [&](int blk) __attribute__((always_inline)) {
+    // The requests for the next block are issued between the matrix instructions of the
+    // first product (an instruction occupies the matrix core for 32 clocks, the wave's issue
+    // slot for a few), column tile by column tile as its W and q^ registers come free;
+    // the second set's 6 + 4*NKW requests are spread over the same loop.
+    auto fetch_wq = [&](int blk, int c) __attribute__((always_inline)) {
         const size_t off = (slot_of(blk) * 4 + wave) * NK * 256 + lane * 4;
-#pragma unroll
-        for (int c = 0; c < NK; c++) {
-            pw[c] = load_f4(Wt + off + c * 256);
-            pq[c] = load_f4(Qt + off + c * 256);
-        }
+        pw[c] = load_f4(Wt + off + c * 256);
+        pq[c] = load_f4(Qt + off + c * 256);
     };
     auto fetch_u = [&](int blk) __attribute__((always_inline)) {
         pu = load_f4(Ut + ((slot_of(blk) * 4 + wave) * NK + blockIdx.y) * 256 + lane * 4);
     };
-    auto fetch_late = [&](Late &p, int blk) __attribute__((always_inline)) {
+    constexpr int NLATE = 6 + 4 * NKW;                 // requests of a Late set
+    constexpr int LATE_PER_C = (NLATE + NK - 1) / NK;  // of which per column tile
+    auto fetch_late = [&](Late &p, int blk, int j) __attribute__((always_inline)) {
         const size_t slot = slot_of(blk);
-#pragma unroll
-        for (int tau = 0; tau < 4; tau++)
-            p.mt[tau] = load_v4(Mt + ((slot * 4 + wave) * 4 + (tau <= wave ? tau : wave)) * 256 + lane * 4);
-        p.el = load_v4(eLc + slot * kC + 16 * wave + 4 * g);
-#pragma unroll
-        for (int kt = 0; kt < NKW; kt++)
-#pragma unroll
-            for (int tau = 0; tau < 4; tau++)
-                p.kd[kt][tau] = load_v4(Kt + ((slot * NK + NKW * wave + kt) * 4 + tau) * 256 + lane * 4);
-        p.elc = eLc[slot * kC + kC - 1];
+        if (j < 4) p.mt[j] = load_v4(Mt + ((slot * 4 + wave) * 4 + (j <= wave ? j : wave)) * 256 + lane * 4);
+        else if (j == 4) p.el = load_v4(eLc + slot * kC + 16 * wave + 4 * g);
+        else if (j == 5) p.elc = eLc[slot * kC + kC - 1];
+        else if (j < NLATE) {
+            const int kt = (j - 6) / 4, tau = (j - 6) % 4;
+            p.kd[kt][tau] = load_v4(Kt + ((slot * NK + NKW * wave + kt) * 4 + tau) * 256 + lane * 4);
+        }
     };
     auto block = [&](int blk, const Late &cur, Late &nxt) __attribute__((always_inline)) {
         const int t0 = blk * kC;
@@ -330,13 +330,14 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
         for (int c = 0; c < NK; c++) {
             p1 = mfma4(pw[c], as_f4(st[c]), p1);
             p2 = mfma4(pq[c], as_f4(st[c]), p2);
+            fetch_wq(blk + 1, c);
+#pragma unroll
+            for (int u = 0; u < LATE_PER_C; u++) fetch_late(nxt, blk + 1, c * LATE_PER_C + u);
         }
-        fetch_wq(blk + 1);
         // ---- D = U - W S0^T: lane (n, g) holds tokens 16w+4g+i of state row row0+n ----
         wy_f32x4 d;
         d[0] = pu.x - p1[0]; d[1] = pu.y - p1[1]; d[2] = pu.z - p1[2]; d[3] = pu.w - p1[3];
         fetch_u(blk + 1);
-        fetch_late(nxt, blk + 1);
         s_d[wave][lane] = d;
         __syncthreads();
         // ---- O = diag(e^L) Q S0^T + M D ------------------------------------------------
@@ -372,9 +373,11 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
         for (int c = 0; c < NK; c++) st[c] = s_st[c][lane];
     };
     Late la, lb;
-    fetch_wq(0);
+#pragma unroll
+    for (int c = 0; c < NK; c++) fetch_wq(0, c);
     fetch_u(0);
-    fetch_late(la, 0);
+#pragma unroll
+    for (int j = 0; j < NLATE; j++) fetch_late(la, 0, j);
     for (int blk = 0; blk < nblk; blk += 2) {
         block(blk, la, lb);
         if (blk + 1 < nblk) block(blk + 1, lb, la);  // uniform over the workgroup
