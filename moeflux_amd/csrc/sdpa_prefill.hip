@@ -28,37 +28,38 @@ __device__ inline float fast_sigmoid(float x) {
 // stay below 2^8, which costs nothing in f32 and spares most rescaling passes.
 static constexpr float kLazyRescale = 8.0f;
 
-// grid (workgroups of 4*RG row groups, Hkv), 256*KS threads.  Waves 4*ks .. 4*ks+3 form
-// set ks: all sets serve the same 4*RG row groups, set ks taking blocks ks, ks + KS, ...
+// grid (workgroups of RW*RG row groups, Hkv), 64*RW*KS threads.  Waves RW*ks .. RW*ks+RW-1
+// form set ks: all sets serve the same RW*RG row groups, set ks taking blocks ks, ks + KS, ...
 // (more waves per SIMD when the rows alone cannot provide them); sets are merged
 // through LDS at the end.
-template <typename KV, int D, int RG, int DEPTH, int KS>
-__global__ __launch_bounds__(256 * KS) void sdpa_prefill_kernel(
+template <typename KV, int D, int RG, int DEPTH, int KS, int RW>
+__global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
     const float *__restrict__ q, const float *__restrict__ gate, int hpk, int Hq, int n_tok,
     int64_t kv_len0, float qscale, float *__restrict__ out) {
     using W = Wave<KV, D>;
     constexpr int NLOAD = W::NLOAD, NACC = W::NACC, NX = W::NX;
     constexpr int BLK_U4 = (NLOAD + NACC) * 64;  // 16-byte words of one block's K and V
-    constexpr int PER_T = BLK_U4 / 256;
-    constexpr int K_T = NLOAD * 64 / 256;        // of which K
-    static_assert(NLOAD % 4 == 0 && NACC % 4 == 0, "a block's K and V are whole 4 KiB units");
+    constexpr int SET = 64 * RW;                 // threads of a wave set
+    constexpr int PER_T = BLK_U4 / SET;
+    constexpr int K_T = NLOAD * 64 / SET;        // of which K
+    static_assert(NLOAD % RW == 0 && NACC % RW == 0, "a set's threads copy whole rounds of a block's K and of its V");
     static_assert(DEPTH == 2 || DEPTH == 4, "the pipeline is written out for two or four stages");
-    static_assert(KS == 1 || (RG == 1 && 4 * 64 * NACC <= 2 * BLK_U4), "the merge reuses the staging buffers");
+    static_assert(KS == 1 || (KS - 1) * RW * RG * NACC * 64 <= 2 * KS * BLK_U4, "the merge reuses the staging buffers");
     __shared__ uint4 kv[2][KS][BLK_U4];
-    __shared__ float s_m[KS][4][16], s_l[KS][4][16];
+    __shared__ float s_m[KS][RW][RG][16], s_l[KS][RW][RG][16];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int rw = wave & 3, ks = wave >> 2, tid = threadIdx.x & 255;
+    const int rw = wave % RW, ks = wave / RW, tid = threadIdx.x % SET;
     const int n = lane & 15, g = lane >> 4;
     const int kvh = blockIdx.y, wg = blockIdx.x;
-    const int hg0 = (wg * 4 + rw) * RG;  // this wave's first row group
+    const int hg0 = (wg * RW + rw) * RG;  // this wave's first row group
     const int64_t blk_elems = (int64_t)W::BLK * D;
     const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
     const KV *vplane = v_tiled + (size_t)kvh * plane_elems;
 
     // blocks the workgroup walks: up to the last position its last row sees
-    const RowGroup wg_last{kvh, wg * 4 * RG + 4 * RG - 1, hpk, Hq, n_tok, kv_len0};
+    const RowGroup wg_last{kvh, wg * RW * RG + RW * RG - 1, hpk, Hq, n_tok, kv_len0};
     const int64_t nblk = (wg_last.limit_max() + W::BLK - 1) / W::BLK;
     const int64_t nit = (nblk + KS - 1) / KS;  // iterations: set ks computes block it * KS + ks
 
@@ -74,12 +75,12 @@ __global__ __launch_bounds__(256 * KS) void sdpa_prefill_kernel(
         const uint4 *kp = (const uint4 *)(kplane + blk * blk_elems) + tid;
         const uint4 *vp = (const uint4 *)(vplane + blk * blk_elems) + tid;
 #pragma unroll
-        for (int i = 0; i < PER_T; i++) stage[s0 + i] = vec_load(i < K_T ? kp + i * 256 : vp + (i - K_T) * 256);
+        for (int i = 0; i < PER_T; i++) stage[s0 + i] = vec_load(i < K_T ? kp + i * SET : vp + (i - K_T) * SET);
     };
     auto commit = [&](int buf, auto st) __attribute__((always_inline)) {
         constexpr int s0 = st.value * PER_T;
 #pragma unroll
-        for (int i = 0; i < PER_T; i++) kv[buf][ks][i * 256 + tid] = stage[s0 + i];
+        for (int i = 0; i < PER_T; i++) kv[buf][ks][i * SET + tid] = stage[s0 + i];
     };
 
     fetch(std::integral_constant<int, 0>{}, 0);
@@ -192,46 +193,53 @@ __global__ __launch_bounds__(256 * KS) void sdpa_prefill_kernel(
 #undef MFA_STEP
     }
 
-    // ---- merge the sets (RG == 1): set 0 takes in the others ------------------------
+    // ---- merge the sets: set 0 takes in the others ----------------------------------
     if constexpr (KS > 1) {
         __syncthreads();  // every wave is done with the staging buffers
-        float4 *xo = reinterpret_cast<float4 *>(&kv[0][0][0]);  // [set - 1][row wave][tile][lane]
-        float l = l_run[0];
-        l += lane_xor(l, 16);
-        l += lane_xor(l, 32);
-        l_run[0] = l;
-        if (ks > 0) {
-            if (g == 0) {
-                s_m[ks][rw][n] = m_ref[0];
-                s_l[ks][rw][n] = l;
-            }
+        float4 *xo = reinterpret_cast<float4 *>(&kv[0][0][0]);  // [set - 1][row wave][group][tile][lane]
 #pragma unroll
-            for (int t = 0; t < NACC; t++)
-                xo[(((ks - 1) * 4 + rw) * NACC + t) * 64 + lane] = float4{o[0][t][0], o[0][t][1], o[0][t][2], o[0][t][3]};
+        for (int r = 0; r < RG; r++) {
+            float l = l_run[r];
+            l += lane_xor(l, 16);
+            l += lane_xor(l, 32);
+            l_run[r] = l;
+            if (ks > 0) {
+                if (g == 0) {
+                    s_m[ks][rw][r][n] = m_ref[r];
+                    s_l[ks][rw][r][n] = l;
+                }
+#pragma unroll
+                for (int t = 0; t < NACC; t++)
+                    xo[((((ks - 1) * RW + rw) * RG + r) * NACC + t) * 64 + lane] =
+                        float4{o[r][t][0], o[r][t][1], o[r][t][2], o[r][t][3]};
+            }
         }
         __syncthreads();
         if (ks > 0) return;
-        float m_all = m_ref[0];
 #pragma unroll
-        for (int j = 1; j < KS; j++) m_all = fmaxf(m_all, s_m[j][rw][n]);
-        const float ref = (m_all == neg_inf()) ? 0.f : m_all;
-        const float a0 = fast_exp2(m_ref[0] - ref);
-        l = l * a0;
+        for (int r = 0; r < RG; r++) {
+            float m_all = m_ref[r];
 #pragma unroll
-        for (int t = 0; t < NACC; t++) {
-            o[0][t][0] *= a0; o[0][t][1] *= a0; o[0][t][2] *= a0; o[0][t][3] *= a0;
-        }
-#pragma unroll
-        for (int j = 1; j < KS; j++) {
-            const float aj = fast_exp2(s_m[j][rw][n] - ref);
-            l += aj * s_l[j][rw][n];
+            for (int j = 1; j < KS; j++) m_all = fmaxf(m_all, s_m[j][rw][r][n]);
+            const float ref = (m_all == neg_inf()) ? 0.f : m_all;
+            const float a0 = fast_exp2(m_ref[r] - ref);
+            float l = l_run[r] * a0;
 #pragma unroll
             for (int t = 0; t < NACC; t++) {
-                const float4 v = xo[(((j - 1) * 4 + rw) * NACC + t) * 64 + lane];
-                o[0][t][0] += aj * v.x; o[0][t][1] += aj * v.y; o[0][t][2] += aj * v.z; o[0][t][3] += aj * v.w;
+                o[r][t][0] *= a0; o[r][t][1] *= a0; o[r][t][2] *= a0; o[r][t][3] *= a0;
             }
+#pragma unroll
+            for (int j = 1; j < KS; j++) {
+                const float aj = fast_exp2(s_m[j][rw][r][n] - ref);
+                l += aj * s_l[j][rw][r][n];
+#pragma unroll
+                for (int t = 0; t < NACC; t++) {
+                    const float4 v = xo[((((j - 1) * RW + rw) * RG + r) * NACC + t) * 64 + lane];
+                    o[r][t][0] += aj * v.x; o[r][t][1] += aj * v.y; o[r][t][2] += aj * v.z; o[r][t][3] += aj * v.w;
+                }
+            }
+            l_run[r] = l;
         }
-        l_run[0] = l;
     } else {
 #pragma unroll
         for (int r = 0; r < RG; r++) {
@@ -242,22 +250,26 @@ __global__ __launch_bounds__(256 * KS) void sdpa_prefill_kernel(
         }
     }
 
-    // ---- normalise, gate, store ---------------------------------------------------
+    // ---- normalise, gate, store (all of the gate is requested before the first use) ----
 #pragma unroll
     for (int r = 0; r < RG; r++) {
         const RowGroup rows{kvh, hg0 + r, hpk, Hq, n_tok, kv_len0};
-        if (!rows.valid(n)) continue;
+        const bool ok = rows.valid(n);
+        const size_t base = (ok ? rows.q_row(n) : 0) * D + 4 * g;
+        uint4 gt[NACC];
+#pragma unroll
+        for (int t = 0; t < NACC; t++) gt[t] = vec_load((const uint4 *)(gate + base + 16 * t));
+        if (!ok) continue;
         const float inv = 1.0f / l_run[r];
-        const size_t base = rows.q_row(n) * D + 4 * g;
 #pragma unroll
         for (int t = 0; t < NACC; t++) {
             // tile t, lane group g, element i is channel 16 t + 4 g + i of row n
-            const float4 gt = *(const float4 *)(gate + base + 16 * t);
+            const float4 gv = __builtin_bit_cast(float4, gt[t]);
             float4 y;
-            y.x = o[r][t][0] * inv * fast_sigmoid(gt.x);
-            y.y = o[r][t][1] * inv * fast_sigmoid(gt.y);
-            y.z = o[r][t][2] * inv * fast_sigmoid(gt.z);
-            y.w = o[r][t][3] * inv * fast_sigmoid(gt.w);
+            y.x = o[r][t][0] * inv * fast_sigmoid(gv.x);
+            y.y = o[r][t][1] * inv * fast_sigmoid(gv.y);
+            y.z = o[r][t][2] * inv * fast_sigmoid(gv.z);
+            y.w = o[r][t][3] * inv * fast_sigmoid(gv.w);
             *(float4 *)(out + base + 16 * t) = y;
         }
     }
@@ -284,29 +296,35 @@ int launch_sdpa_prefill(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D
         return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld for %d tokens)", (long long)kv_len, n_tok);
     const int hpk = Hq / Hkv;
     const int64_t nhg = ((int64_t)n_tok * hpk + 15) / 16;
-    // Two row groups per wave once that still leaves every CU two workgroups; two wave sets
-    // per workgroup when the rows do not even give every CU two single-set workgroups.
-    const int rg = ((nhg + 7) / 8 * Hkv >= 2 * (int64_t)num_cus && D <= 128) ? 2 : 1;
-    const int ks = (rg == 1 && D <= 128 && (nhg + 3) / 4 * Hkv < 2 * (int64_t)num_cus) ? 2 : 1;
-    const int64_t nwg = (nhg + 4 * rg - 1) / (4 * rg);
+    // Shapes of a workgroup (row waves RW x row groups per wave RG x wave sets KS):
+    //   large chunks  4 x 2 x 1: two row groups per wave share each operand read from LDS;
+    //   medium        4 x 1 x 1 (every CU still gets two workgroups);
+    //   small (the rows alone would leave a wave alone on its SIMD)  4 x 1 x 2: the blocks are
+    //   split over two wave sets.  (2 x 2 x 2, four waves with two row groups each, was
+    //   measured 35 % slower at 512 tokens: the two groups' instructions do not interleave;
+    //   2 x 1 x 2, two small workgroups per CU, 15 % slower.)
+    const bool big = (nhg + 7) / 8 * Hkv >= 2 * (int64_t)num_cus && D <= 128;
+    const bool small = !big && D <= 128 && (nhg + 3) / 4 * Hkv < 2 * (int64_t)num_cus;
+    const int rw = 4, rg = big ? 2 : 1;
+    const int64_t nwg = (nhg + rw * rg - 1) / (rw * rg);
     if (nwg > 0x7fffffff || Hkv > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     const int64_t kv_len0 = kv_len - n_tok;
     const dim3 grid((unsigned)nwg, Hkv);
-#define MFA_LAUNCH(KV, DD, RGG, KSS)                                                                  \
-    hipLaunchKernelGGL((sdpa_prefill_kernel<KV, DD, RGG, (DD <= 128 && RGG == 1) ? 4 : 2, KSS>), grid, \
-                       dim3(256 * KSS), 0, stream, (const KV *)k_tiled, (const KV *)v_tiled, plane_elems, q, \
-                       gate, hpk, Hq, n_tok, kv_len0, qscale, out)
+#define MFA_LAUNCH(KV, DD, RGG, DEP, KSS, RWW)                                                                 \
+    hipLaunchKernelGGL((sdpa_prefill_kernel<KV, DD, RGG, DEP, KSS, RWW>), grid, dim3(64 * RWW * KSS), 0, stream, \
+                       (const KV *)k_tiled, (const KV *)v_tiled, plane_elems, q, gate, hpk, Hq, n_tok, kv_len0,   \
+                       qscale, out)
 #define MFA_LAUNCH_D(KV)                                         \
-    if (D == 256) MFA_LAUNCH(KV, 256, 1, 1);                     \
+    if (D == 256) MFA_LAUNCH(KV, 256, 1, 2, 1, 4);               \
     else if (D == 128) {                                         \
-        if (rg == 2) MFA_LAUNCH(KV, 128, 2, 1);                  \
-        else if (ks == 2) MFA_LAUNCH(KV, 128, 1, 2);             \
-        else MFA_LAUNCH(KV, 128, 1, 1);                          \
+        if (big) MFA_LAUNCH(KV, 128, 2, 2, 1, 4);                \
+        else if (small) MFA_LAUNCH(KV, 128, 1, 4, 2, 4);         \
+        else MFA_LAUNCH(KV, 128, 1, 4, 1, 4);                    \
     } else {                                                     \
-        if (rg == 2) MFA_LAUNCH(KV, 64, 2, 1);                   \
-        else if (ks == 2) MFA_LAUNCH(KV, 64, 1, 2);              \
-        else MFA_LAUNCH(KV, 64, 1, 1);                           \
+        if (big) MFA_LAUNCH(KV, 64, 2, 2, 1, 4);                 \
+        else if (small) MFA_LAUNCH(KV, 64, 1, 4, 2, 4);          \
+        else MFA_LAUNCH(KV, 64, 1, 4, 1, 4);                     \
     }
     if (kv_dtype == MFA_KV_BF16) { MFA_LAUNCH_D(uint16_t) } else { MFA_LAUNCH_D(float) }
 #undef MFA_LAUNCH_D
