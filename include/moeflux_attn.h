@@ -150,6 +150,32 @@ int mfa_dequant_matvec_4bit(int32_t out_dim, int32_t in_dim, int32_t group_size,
                             const uint32_t *w_packed, const uint16_t *scales,
                             const uint16_t *biases, const float *x, float *out);
 
+/* ---- attention over a latent cache (multi-head latent attention, folded) ------ */
+
+/* Replaces mla_sdpa_folded and its tiled form mla_sdpa_tile_accumulate /
+ * mla_sdpa_tile_finalize (shaders.metal:1688-1987; encoders
+ * gpu_mla.rs:146-200 encode_mla_sdpa_folded and :202 encode_mla_sdpa_folded_tiled;
+ * call site mla_attn_forward.rs:462-476) at every cache_len >= 1, one launch pair whatever the
+ * length: per head h, scores (q_prime[h] . latent[t] + q_pe[h] . rope_k[t]) *
+ * softmax_scale over t in [0, cache_len), softmax, v_combine[h] = sum_t w[t]
+ * latent[t].  All f32, all on the device, on the context's stream:
+ *   q_prime, v_combine [num_heads, kv_lora_rank]; q_pe [num_heads, qk_rope_head_dim];
+ *   latent_cache [cache_len, kv_lora_rank]; rope_k_cache [cache_len, qk_rope_head_dim].
+ * Built for kv_lora_rank 512, qk_rope_head_dim 64 (variants.rs, the MLA variants);
+ * other widths return MFA_ERR_SHAPE.  The context supplies the stream and the
+ * split workspace; its own layers and caches are not touched. */
+int mfa_mla_sdpa_folded_dev(mfa_ctx *ctx, int32_t num_heads, int32_t kv_lora_rank,
+                            int32_t qk_rope_head_dim, int32_t cache_len, float softmax_scale,
+                            const float *q_prime_dev, const float *q_pe_dev,
+                            const float *latent_cache_dev, const float *rope_k_cache_dev,
+                            float *v_combine_dev);
+/* Stateless host-pointer twin (the shape of the reference's test harness,
+ * tests/mla_sdpa_tiled.rs:84-140): uploads, runs the same kernels, downloads. */
+int mfa_mla_sdpa_folded(int32_t num_heads, int32_t kv_lora_rank, int32_t qk_rope_head_dim,
+                        int32_t cache_len, float softmax_scale, const float *q_prime,
+                        const float *q_pe, const float *latent_cache, const float *rope_k_cache,
+                        float *v_combine);
+
 /* ---- what precedes the attention core in a full-attention layer -------------- */
 
 /* Per-layer constants of the prologue: the bf16 weights of the per-head RMS

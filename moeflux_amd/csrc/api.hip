@@ -763,6 +763,77 @@ int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on) {
     return MFA_OK;
 }
 
+/* ---- attention over a latent cache -------------------------------------------------- */
+
+static int ensure_workspace_elems(Ctx *c, size_t need_o, size_t need_ml) {
+    if (need_o <= c->part_o_elems && need_ml <= c->part_ml_elems) return MFA_OK;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    if (need_o > c->part_o_elems) {
+        if (c->part_o) MFA_HIP(hipFree(c->part_o));
+        c->part_o = nullptr;
+        c->part_o_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->part_o, need_o * sizeof(float)));
+        c->part_o_elems = need_o;
+    }
+    if (need_ml > c->part_ml_elems) {
+        if (c->part_ml) MFA_HIP(hipFree(c->part_ml));
+        c->part_ml = nullptr;
+        c->part_ml_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->part_ml, need_ml * sizeof(float)));
+        c->part_ml_elems = need_ml;
+    }
+    return MFA_OK;
+}
+
+static int mla_check(int32_t H, int32_t R, int32_t P, int32_t L) {
+    if (H <= 0 || R <= 0 || P <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");
+    if (L <= 0) return fail(MFA_ERR_INVALID, "cache_len must be > 0 (got %d)", L);
+    if (!mla_shape_supported(R, P))
+        return fail(MFA_ERR_SHAPE, "kv_lora_rank %d / qk_rope_head_dim %d not supported (512 / 64)", R, P);
+    return MFA_OK;
+}
+
+int mfa_mla_sdpa_folded_dev(mfa_ctx *ctx, int32_t num_heads, int32_t kv_lora_rank, int32_t qk_rope_head_dim,
+                            int32_t cache_len, float softmax_scale, const float *q_prime, const float *q_pe,
+                            const float *latent_cache, const float *rope_k_cache, float *v_combine) {
+    Ctx *c = as_ctx(ctx);
+    if (!c || !q_prime || !q_pe || !latent_cache || !rope_k_cache || !v_combine)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    MFA_TRY(mla_check(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len));
+    const MlaPlan plan = mla_plan(num_heads, cache_len, c->num_cus);
+    MFA_TRY(ensure_workspace_elems(c, mla_workspace_o_elems(plan, kv_lora_rank), mla_workspace_ml_elems(plan)));
+    return launch_mla_sdpa_folded(c->stream, num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale,
+                                  q_prime, q_pe, latent_cache, rope_k_cache, v_combine, workspace(c), plan);
+}
+
+int mfa_mla_sdpa_folded(int32_t num_heads, int32_t kv_lora_rank, int32_t qk_rope_head_dim, int32_t cache_len,
+                        float softmax_scale, const float *q_prime, const float *q_pe, const float *latent_cache,
+                        const float *rope_k_cache, float *v_combine) {
+    if (!q_prime || !q_pe || !latent_cache || !rope_k_cache || !v_combine)
+        return fail(MFA_ERR_INVALID, "NULL argument");
+    MFA_TRY(mla_check(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len));
+    const size_t H = num_heads, R = kv_lora_rank, P = qk_rope_head_dim, L = cache_len;
+    int dev = 0;
+    hipDeviceProp_t prop;
+    MFA_HIP(hipGetDevice(&dev));
+    MFA_HIP(hipGetDeviceProperties(&prop, dev));
+    const MlaPlan plan = mla_plan(num_heads, cache_len, prop.multiProcessorCount);
+    DevBuf dq, dp, dl, dr, dout, dpo, dml;
+    MFA_TRY(dq.upload(q_prime, H * R * 4));
+    MFA_TRY(dp.upload(q_pe, H * P * 4));
+    MFA_TRY(dl.upload(latent_cache, L * R * 4));
+    MFA_TRY(dr.upload(rope_k_cache, L * P * 4));
+    MFA_TRY(dout.alloc(H * R * 4));
+    const size_t no = mla_workspace_o_elems(plan, kv_lora_rank), nml = mla_workspace_ml_elems(plan);
+    MFA_TRY(dpo.alloc(no * 4));
+    MFA_TRY(dml.alloc(nml * 4));
+    const SdpaWorkspace ws{dpo.as<float>(), dml.as<float>(), no, nml};
+    MFA_TRY(launch_mla_sdpa_folded(nullptr, num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale,
+                                   dq.as<float>(), dp.as<float>(), dl.as<float>(), dr.as<float>(), dout.as<float>(),
+                                   ws, plan));
+    return dout.download(v_combine, H * R * 4);
+}
+
 /* ---- projections ------------------------------------------------------------------- */
 
 int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs) {

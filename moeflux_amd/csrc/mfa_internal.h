@@ -186,6 +186,24 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
                 int forced_splits, int partial_only = 0);
+// Log-sum-exp merge of partials laid out [kv head][16-row group][split][16][D] (+ (max, sum) per row),
+// normalisation, and the sigmoid gate when `gate` is not null.  out, gate: [n_tok, Hq*D].
+int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,
+                      int n_tok, const float *gate, float *out);
+// mla_sdpa.hip: one query token of H heads against a latent cache [L, R] + rotary keys [L, P].
+struct MlaPlan {
+    int splits;     // workgroups along the cache
+    int bps;        // 16-position blocks per split
+    int nhg;        // 16-head groups
+    int nwg_heads;  // workgroups along the heads (4 groups each)
+};
+bool mla_shape_supported(int kv_lora_rank, int qk_rope_head_dim);
+MlaPlan mla_plan(int H, int L, int num_cus);
+size_t mla_workspace_o_elems(const MlaPlan &p, int R);
+size_t mla_workspace_ml_elems(const MlaPlan &p);
+int launch_mla_sdpa_folded(hipStream_t stream, int H, int R, int P, int L, float softmax_scale,
+                           const float *q_prime, const float *q_pe, const float *latent, const float *rope_k,
+                           float *out, const SdpaWorkspace &ws, const MlaPlan &plan);
 // dequant_matvec.hip: up to 8 four-bit dequantising matrix-vector products in one launch.
 int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const *w, const uint16_t *const *scales,
                                const uint16_t *const *biases, const float *const *x, float *const *out,

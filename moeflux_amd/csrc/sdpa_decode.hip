@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
         rows[r] = (s < nsplit) ? *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0)
                                : float4{0.f, 0.f, 0.f, 0.f};
     }
-    const float gt_in = (tid < 64) ? gate[(size_t)blockIdx.x * D + blockIdx.y * 64 + tid] : 0.f;
+    const float gt_in = (gate && tid < 64) ? gate[(size_t)blockIdx.x * D + blockIdx.y * 64 + tid] : 0.f;
 
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
 #pragma unroll
@@ -309,9 +309,19 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
 #pragma unroll
         for (int x = 0; x < 16; x++) t += ((const float *)&acc4[x][ql])[qc];
         const int d = blockIdx.y * 64 + tid;
-        const float gt = 1.0f / (1.0f + expf(-gt_in));
+        const float gt = gate ? 1.0f / (1.0f + expf(-gt_in)) : 1.0f;
         out[(size_t)blockIdx.x * D + d] = (t / den) * gt;
     }
+}
+
+int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,
+                      int n_tok, const float *gate, float *out) {
+    if (splits < 1 || splits > kMaxSplits || D % 64 != 0)
+        return fail(MFA_ERR_INVALID, "merge: %d splits (1..%d), width %d (multiple of 64)", splits, kMaxSplits, D);
+    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, ws.part_o, ws.part_ml,
+                       splits, hpk, Hq, nhg, D, gate, out);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
 }
 
 bool sdpa_shape_supported(int kv_dtype, int head_dim) {

@@ -422,3 +422,19 @@ def dequant_matvec_4bit_cpu(packed, scales_bf16, biases_bf16, in_dim, out_dim, x
     _chk(lib.mfa_dequant_matvec_4bit(out_dim, in_dim, 64, _p(packed), _p(sc), _p(bi), _p(x), _p(out)),
          "mfa_dequant_matvec_4bit")
     return out
+
+
+def mla_sdpa_folded(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale, q_prime, q_pe,
+                    latent_cache, rope_k_cache):
+    """Attention of one token over a latent cache, the folded form (encode_mla_sdpa_folded,
+    gpu_mla.rs:146-200; kernel shaders.metal:1688-1816), host arrays in and out."""
+    lib = ffi.load()
+    qp = _f32(q_prime, num_heads * kv_lora_rank, "q_prime")
+    qe = _f32(q_pe, num_heads * qk_rope_head_dim, "q_pe")
+    lat = _f32(latent_cache, cache_len * kv_lora_rank, "latent_cache")
+    rk = _f32(rope_k_cache, cache_len * qk_rope_head_dim, "rope_k_cache")
+    out = np.empty(num_heads * kv_lora_rank, dtype=np.float32)
+    _chk(lib.mfa_mla_sdpa_folded(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale,
+                                 _p(qp), _p(qe), _p(lat), _p(rk), _p(out)), "mfa_mla_sdpa_folded")
+    return out
+

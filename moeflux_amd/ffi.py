@@ -61,6 +61,10 @@ SIGNATURES = {
     "mfa_full_attn_step_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_dequant_matvec_4bit_dev": (C.c_int, [vp, C.c_int32, vp]),
     "mfa_dequant_matvec_4bit": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, vp, u16p, u16p, f32p, f32p]),
+    "mfa_mla_sdpa_folded_dev": (C.c_int, [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float,
+                                          f32p, f32p, f32p, f32p, f32p]),
+    "mfa_mla_sdpa_folded": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float,
+                                      f32p, f32p, f32p, f32p, f32p]),
     "mfa_state_size": (C.c_int64, [vp]),
     "mfa_state_save": (C.c_int64, [vp, vp, C.c_int64]),
     "mfa_state_load": (C.c_int, [vp, vp, C.c_int64]),

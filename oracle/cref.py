@@ -293,3 +293,14 @@ def dequant_matvec_4bit(packed, scales_bf16, biases_bf16, in_dim, out_dim, x):
     _check(rc, "orc_dequant_matvec_4bit")
     return out
 
+
+def mla_sdpa_folded(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale, q_prime, q_pe,
+                    latent_cache, rope_k_cache):
+    q_prime, q_pe, latent_cache, rope_k_cache = map(_f32, (q_prime, q_pe, latent_cache, rope_k_cache))
+    out = np.empty(num_heads * kv_lora_rank, dtype=np.float32)
+    rc = lib().orc_mla_sdpa_folded(C.c_int32(num_heads), C.c_int32(kv_lora_rank), C.c_int32(qk_rope_head_dim),
+                                   C.c_int32(cache_len), C.c_float(softmax_scale), _p(q_prime), _p(q_pe),
+                                   _p(latent_cache), _p(rope_k_cache), _p(out))
+    _check(rc, "orc_mla_sdpa_folded")
+    return out
+

@@ -20,7 +20,7 @@
  *   orc_rms_norm_bare, orc_rms_norm_qk, orc_rms_norm_gated, orc_decay_beta,
  *   orc_gated_delta_recurrence, orc_gdn_step, orc_prefill_attn,
  *   orc_prefill_gdn, orc_rms_norm_per_head, orc_apply_rotary_emb,
- *   orc_attn_prologue, orc_dequant_matvec_4bit : pinned by float64 brute force on small shapes, closed
+ *   orc_attn_prologue, orc_dequant_matvec_4bit, orc_mla_sdpa_folded : pinned by float64 brute force on small shapes, closed
  *   forms and invariants (the reference holds no numeric vectors for them).
  *   The Accelerate-BLAS variant of the recurrence (infer.m:4954-4993) is not
  *   restated: parity unpinned at that boundary (mathematically identical to
@@ -572,5 +572,49 @@ ORC_API int orc_dequant_matvec_4bit(const uint32_t *packed, const uint16_t *scal
         }
         out[r] = acc;
     }
+    return 0;
+}
+
+/* ---- attention over a compressed (latent) cache --------------------------------- */
+
+/* crates/moeflux/shaders/shaders.metal:1688-1816 (mla_sdpa_folded; the tiled form
+ * :1818-1987 computes the same function): per head h
+ *   s[t] = (q'[h] . latent[t] + q_pe[h] . rope_k[t]) * softmax_scale   (fma accumulation,
+ *          the latent part first), softmax over t (max, exp, sum, times 1/sum),
+ *   out[h, c] = sum_t s[t] latent[t, c]                                  (fma accumulation).
+ * q_prime, out: [H, R]; q_pe: [H, P]; latent: [L, R]; rope_k: [L, P]. */
+ORC_API int orc_mla_sdpa_folded(int32_t num_heads, int32_t kv_lora_rank, int32_t qk_rope_head_dim,
+                                int32_t cache_len, float softmax_scale, const float *q_prime,
+                                const float *q_pe, const float *latent, const float *rope_k, float *out) {
+    if (!q_prime || !q_pe || !latent || !rope_k || !out) return -1;
+    if (num_heads <= 0 || kv_lora_rank <= 0 || qk_rope_head_dim <= 0 || cache_len <= 0) return -1;
+    const int R = kv_lora_rank, P = qk_rope_head_dim;
+    float *scores = (float *)malloc((size_t)cache_len * sizeof(float));
+    if (!scores) return -1;
+    for (int h = 0; h < num_heads; h++) {
+        const float *qh = q_prime + (int64_t)h * R, *qp = q_pe + (int64_t)h * P;
+        for (int t = 0; t < cache_len; t++) {
+            const float *lt = latent + (int64_t)t * R, *rt = rope_k + (int64_t)t * P;
+            float s = 0.0f;
+            for (int c = 0; c < R; c++) s = fmaf(qh[c], lt[c], s);
+            for (int r = 0; r < P; r++) s = fmaf(qp[r], rt[r], s);
+            scores[t] = s * softmax_scale;
+        }
+        float maxv = -INFINITY;
+        for (int t = 0; t < cache_len; t++) maxv = fmaxf(maxv, scores[t]);
+        float sum = 0.0f;
+        for (int t = 0; t < cache_len; t++) {
+            scores[t] = expf(scores[t] - maxv);
+            sum += scores[t];
+        }
+        const float inv_sum = 1.0f / sum;
+        for (int t = 0; t < cache_len; t++) scores[t] *= inv_sum;
+        for (int c = 0; c < R; c++) {
+            float acc = 0.0f;
+            for (int t = 0; t < cache_len; t++) acc = fmaf(scores[t], latent[(int64_t)t * R + c], acc);
+            out[(int64_t)h * R + c] = acc;
+        }
+    }
+    free(scores);
     return 0;
 }

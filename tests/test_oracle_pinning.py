@@ -410,3 +410,57 @@ def test_dequant_matvec_against_float64_matrix_product():
     e = np.zeros(in_dim, np.float32)
     e[77] = 1.0
     assert np.allclose(cref.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, e), W[:, 77], rtol=1e-6)
+
+
+# ---- attention over a latent cache (MLA, folded form) ---------------------------------
+
+def _mla_inputs(seed, H, R, P, L):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((H, R)).astype(np.float32) * 0.3, rng.standard_normal((H, P)).astype(np.float32) * 0.3,
+            rng.standard_normal((L, R)).astype(np.float32), rng.standard_normal((L, P)).astype(np.float32))
+
+
+@pytest.mark.parametrize("H,R,P,L", [(3, 8, 4, 1), (3, 8, 4, 7), (16, 64, 16, 33), (5, 32, 8, 130)])
+def test_mla_against_float64_softmax(H, R, P, L):
+    from scipy.special import softmax
+    qp, qe, lat, rk = _mla_inputs(L, H, R, P, L)
+    scale = 0.37
+    s = (qp.astype(np.float64) @ lat.astype(np.float64).T + qe.astype(np.float64) @ rk.astype(np.float64).T) * scale
+    want = softmax(s, axis=1) @ lat.astype(np.float64)
+    got = cref.mla_sdpa_folded(H, R, P, L, scale, qp, qe, lat, rk).reshape(H, R)
+    assert rel_err(got, want.astype(np.float32)) <= F32
+
+
+def test_mla_is_multi_query_attention_over_the_concatenated_key():
+    """The folded form is MQA with key [latent | rope_k], value latent, one kv head and no gate:
+    the already pinned orc_sdpa, fed the concatenation (value padded to the key's width, query
+    rescaled to its 1/sqrt(d), gate large so the sigmoid is 1), must agree."""
+    H, R, P, L = 4, 48, 16, 57
+    qp, qe, lat, rk = _mla_inputs(2, H, R, P, L)
+    scale = 0.21
+    d = R + P
+    q = np.concatenate([qp, qe], axis=1) * (scale * np.sqrt(d))
+    k = np.concatenate([lat, rk], axis=1)
+    v = np.concatenate([lat, np.zeros((L, P), np.float32)], axis=1)
+    ref = cref.sdpa(L, H, 1, d, q.astype(np.float32), np.full(H * d, 40.0, np.float32), k, v).reshape(H, d)[:, :R]
+    got = cref.mla_sdpa_folded(H, R, P, L, scale, qp, qe, lat, rk).reshape(H, R)
+    assert rel_err(got, ref) <= 3e-6
+
+
+def test_mla_closed_forms():
+    H, R, P, L = 3, 16, 4, 9
+    qp, qe, lat, rk = _mla_inputs(4, H, R, P, L)
+    f = lambda *a: cref.mla_sdpa_folded(H, R, P, len(a[2]), 0.5, *a).reshape(H, R)
+    # one position: the output is that latent row, whatever the query
+    assert np.allclose(f(qp, qe, lat[:1], rk[:1]), np.broadcast_to(lat[0], (H, R)), rtol=1e-6)
+    # zero query: uniform weights, the mean latent row
+    z = f(qp * 0, qe * 0, lat, rk)
+    assert np.allclose(z, np.broadcast_to(lat.mean(axis=0), (H, R)), atol=2e-7, rtol=1e-5)
+    # only the rope part differs between positions with equal latent rows: output is that row
+    same = np.broadcast_to(lat[0], (L, R)).copy()
+    assert np.allclose(f(qp, qe, same, rk), np.broadcast_to(lat[0], (H, R)), rtol=1e-5, atol=1e-6)
+    # a rope key far along q_pe takes all the weight: this pins that the rope term enters the score
+    rk2 = rk.copy()
+    rk2[5] = 60.0 * qe[1] / np.dot(qe[1], qe[1])
+    out = f(qp * 0, qe, lat, rk2)
+    assert np.allclose(out[1], lat[5], rtol=1e-4, atol=1e-5)
