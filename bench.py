@@ -382,11 +382,15 @@ def bench_mla(steps, warmup, seed, lens=(4096, 32768)):
                 raise RuntimeError(ffi.last_error())
 
         _, ev_ms = _timed(ctx, lib, step, steps, warmup)
-        flops = 2.0 * H * L * (R + P + R)
+        flops = 2.0 * H * L * (R + P + R)        # the two products, once
         alg = L * (R + P) * 4 + 2 * H * R * 4 + H * P * 4
-        res[f"L{L}"] = {"us_per_call": ev_ms * 1e3, "flops": flops, "tflops": flops / (ev_ms * 1e-3) / 1e12,
-                        "pct_f32_mfma_peak": 100.0 * flops / (ev_ms * 1e-3) / 1e12 / 157.3,
-                        "algorithmic_bytes": alg, "gbps": alg / (ev_ms * 1e-3) / 1e9}
+        sec = ev_ms * 1e-3
+        res[f"L{L}"] = {"us_per_call": ev_ms * 1e3, "flops": flops, "tflops": flops / sec / 1e12,
+                        # every product is three bf16 partial products on the matrix pipeline
+                        "bf16_mfma_flops_issued": 3 * flops,
+                        "pct_bf16_mfma_peak": 100.0 * 3 * flops / sec / 1e12 / 2500.0,
+                        "algorithmic_bytes": alg, "gbps": alg / sec / 1e9,
+                        "pct_hbm_peak": 100.0 * alg / sec / 1e9 / HBM_PEAK_GBPS}
         for lat, rk in sets:
             lat.free(); rk.free()
     ctx.close()
