@@ -7,15 +7,21 @@
 // and bias per 64 inputs.
 //
 // Bound: HBM, 0.5625 bytes per weight (4 bits + 2 x bf16 per 64).  At that rate the VALU
-// work per weight matters (16 T weights/s at 8 TB/s against 39 T lane-instructions/s): per
-// u32 the kernel spends two masks, eight byte->float conversions and eight FMAs, using
-//   sum (n s + b) x = s sum n x + b sum x
-// so scale and bias are applied once per lane and row, and the high nibbles are converted as
-// 16 n against x/16 (exact) to save their shift.
-//
-// A wave owns a run of rows.  Lane l always handles the same 16-byte column chunks
-// (l, l+64, ...), so its slice of x (32 floats per chunk) and the slice's sum stay in
-// registers for all of the wave's rows; a row's weights are requested one row ahead.
+// work per weight matters (16 T weights/s at 8 TB/s against 39 T lane-instructions/s), so the
+// multiply-adds run on the matrix pipeline and the vector ALU only converts:
+//   * A nibble n becomes the bf16 number 1 + n/16 (exponent bits of 1.0, n in the top four
+//     mantissa bits): two nibbles per shift + and-or, exact, one instruction per weight.
+//   * x is split into three bf16 parts by truncation (x = h + m + l exactly), which sit in
+//     three columns of the B operand; a 16x16x32 instruction therefore gives, per row,
+//     sum (1 + n/16) x exactly up to f32 accumulation.
+//   * One instruction covers 32 inputs per lane group, i.e. two scale groups of 64 per four
+//     instructions: columns 0..2 carry the first group's x (zero elsewhere), columns 3..5 the
+//     second's, so the two groups' sums stay apart in one accumulator tile.
+//   * Per group g and row r:  out += 16 s (D - X_g) + b X_g  with X_g = sum x over the group;
+//     D is about 1.5 X_g, so the subtraction costs no more than two bits.
+// A workgroup owns 16 rows (the M side of the tile); its waves split the inputs in runs of
+// 1024, each lane requesting its 8 x 16 bytes of weights before anything else, and x, the
+// scales and the biases are staged in LDS while those requests are in flight.
 #include <type_traits>
 
 #include "gdn_device.h"
@@ -36,99 +42,159 @@ struct MatvecSpecs {
 
 typedef unsigned int mv_u32x4 __attribute__((ext_vector_type(4)));
 
-template <int N, typename F> __device__ __forceinline__ void mv_static_for(F &&f) {
-    if constexpr (N > 0) {
-        mv_static_for<N - 1>(f);
-        f(std::integral_constant<int, N - 1>{});
-    }
-}
+typedef __attribute__((ext_vector_type(8))) __bf16 mv_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float mv_f32x4;
 
-// sum over the 8 nibbles of `w` of nibble * x: low nibbles of each byte against xl, high
-// nibbles (left in place, i.e. 16 * nibble) against xh = x / 16.
-__device__ inline float dot8(uint32_t w, const float *xl, const float *xh, float acc) {
-    uint32_t lo = w & 0x0F0F0F0Fu, hi = w & 0xF0F0F0F0u;
-    // keep the two masked words as they are: the byte selects below then map onto
-    // v_cvt_f32_ubyte0..3 (one instruction per nibble) instead of a bit-field extract each
-    asm volatile("" : "+v"(lo), "+v"(hi));
-    acc = fmaf((float)(lo & 0xFFu), xl[0], acc);
-    acc = fmaf((float)(hi & 0xFFu), xh[0], acc);
-    acc = fmaf((float)((lo >> 8) & 0xFFu), xl[1], acc);
-    acc = fmaf((float)((hi >> 8) & 0xFFu), xh[1], acc);
-    acc = fmaf((float)((lo >> 16) & 0xFFu), xl[2], acc);
-    acc = fmaf((float)((hi >> 16) & 0xFFu), xh[2], acc);
-    acc = fmaf((float)(lo >> 24), xl[3], acc);
-    acc = fmaf((float)(hi >> 24), xh[3], acc);
-    return acc;
-}
+struct MatvecTiles {
+    int first[kMvMaxSpecs + 1];  // first 16-row tile of every product, and the total
+};
 
-// grid (ceil(max out_dim / (4 * ROWS)), n_specs), 256 threads; NCH = ceil(in_dim / 2048).
-template <int NCH, int ROWS>
-__global__ __launch_bounds__(256) void dequant_matvec_4bit_kernel(MatvecSpecs sp) {
-    const int s = blockIdx.y;
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void dequant_matvec_mfma_kernel(MatvecSpecs sp, MatvecTiles tl, int n_specs) {
+    constexpr int NTHR = WAVES * 64;
+    constexpr int KP = WAVES * 1024;   // inputs covered by the workgroup (in_dim padded)
+    constexpr int G = KP / 64;         // scale groups
+    constexpr int STEPS = 8;           // 128-input steps per wave
+    __shared__ __attribute__((aligned(16))) uint16_t xs[3][KP];       // bf16 parts of x; within a run of 8 inputs the order is 0,4,1,5,2,6,3,7
+    __shared__ __attribute__((aligned(16))) uint16_t zeros[128 * STEPS + 128];  // what the other lanes of the B operand read
+    // scales and biases of the tile's rows as stored (bf16), [group][row]; + 4: the staging writes walk the groups
+    __shared__ __attribute__((aligned(8))) uint16_t sc_l[G][16 + 4], bi_l[G][16 + 4];
+    __shared__ float xsum[G];
+    __shared__ __attribute__((aligned(16))) float red[WAVES][16];
+
+    int s = 0;
+    while (s + 1 < n_specs && (int)blockIdx.x >= tl.first[s + 1]) s++;
+    const int row0 = ((int)blockIdx.x - tl.first[s]) * 16;
     const int in_dim = sp.in_dim[s], out_dim = sp.out_dim[s];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int row0 = (blockIdx.x * 4 + wave) * ROWS;
-    if (row0 >= out_dim) return;
-    const int n16 = in_dim >> 5;  // 16-byte chunks (32 inputs) per row
-    const int groups = in_dim >> 6;
-    const uint32_t *W = sp.w[s];
-    const uint16_t *S = sp.scales[s], *B = sp.biases[s];
-    const float *x = sp.x[s];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int nchunk = in_dim >> 5, groups = in_dim >> 6, words = in_dim >> 3;
 
-    // this lane's slice of x: even inputs (low nibbles) as they are, odd inputs / 16
-    float xl[NCH][16], xh[NCH][16], sumx[NCH];
-    bool live[NCH];
+    // ---- weights: row n of the tile, 32-input chunk 4 S + g of step S; all requested now ----
+    mv_u32x4 w[STEPS];
+    {
+        const uint32_t *wrow = sp.w[s] + (size_t)min(row0 + n, out_dim - 1) * words;
 #pragma unroll
-    for (int c = 0; c < NCH; c++) {
-        const int ch = lane + 64 * c;
-        live[c] = ch < n16;
-        sumx[c] = 0.f;
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            float4 v = {0.f, 0.f, 0.f, 0.f};
-            if (live[c]) v = load_f4(x + (size_t)ch * 32 + 4 * u);
-            // word u/2 of the chunk, bytes 2(u%2) and 2(u%2)+1: inputs 8(u/2) + 4(u%2) + {0,1,2,3}
-            xl[c][2 * u] = v.x;
-            xh[c][2 * u] = v.y * 0.0625f;
-            xl[c][2 * u + 1] = v.z;
-            xh[c][2 * u + 1] = v.w * 0.0625f;
-            sumx[c] += (v.x + v.y) + (v.z + v.w);
+        for (int st = 0; st < STEPS; st++) {
+            const int c = 4 * (wave * STEPS + st) + g;
+            w[st] = *reinterpret_cast<const mv_u32x4 *>(wrow + (c < nchunk ? c : 0) * 4);  // past the row: any chunk, x is 0 there
         }
     }
-    auto fetch = [&](int r, mv_u32x4 (&w)[NCH], float (&sc)[NCH], float (&bi)[NCH]) __attribute__((always_inline)) {
-        if (r > out_dim - 1) r = out_dim - 1;  // past the end: re-read the last row, never stored
+    // ---- stage x (a run of 8 inputs per thread and pass), the scales and the biases; every
+    //      request first, so that the workgroup pays one round trip, not one per pass ----
+    {
+        constexpr int XP = KP / 8 / NTHR;       // passes over x
+        constexpr int SP = 16 * G / NTHR;   // passes over the (row, group) pairs
+        const float *x = sp.x[s];
+        const uint16_t *S = sp.scales[s], *B = sp.biases[s];
+        float4 xa[XP], xb4[XP];
+        uint16_t sraw[SP], braw[SP];
 #pragma unroll
-        for (int c = 0; c < NCH; c++) {
-            const int ch = live[c] ? lane + 64 * c : 0;
-            w[c] = *reinterpret_cast<const mv_u32x4 *>(W + (size_t)r * (in_dim >> 3) + (size_t)ch * 4);
-            sc[c] = bf16_bits_to_f32(S[(size_t)r * groups + (ch >> 1)]);
-            bi[c] = bf16_bits_to_f32(B[(size_t)r * groups + (ch >> 1)]);
+        for (int p = 0; p < XP; p++) {
+            const int r = tid + p * NTHR;
+            const int at = 8 * r < in_dim ? 8 * r : 0;
+            xa[p] = load_f4(x + at);
+            xb4[p] = load_f4(x + at + 4);
         }
-    };
-    auto row = [&](int r, const mv_u32x4 (&w)[NCH], const float (&sc)[NCH], const float (&bi)[NCH]) __attribute__((always_inline)) {
-        float tot = 0.f;
 #pragma unroll
-        for (int c = 0; c < NCH; c++) {
-            const float a0 = dot8(w[c][0], &xl[c][0], &xh[c][0], 0.f);
-            const float a1 = dot8(w[c][1], &xl[c][4], &xh[c][4], 0.f);
-            const float a2 = dot8(w[c][2], &xl[c][8], &xh[c][8], 0.f);
-            const float a3 = dot8(w[c][3], &xl[c][12], &xh[c][12], 0.f);
-            const float part = fmaf(sc[c], (a0 + a1) + (a2 + a3), bi[c] * sumx[c]);
-            tot += live[c] ? part : 0.f;
+        for (int p = 0; p < SP; p++) {
+            const int i = tid + p * NTHR;
+            const int r = i / G, gg = i % G;
+            const size_t at = (size_t)min(row0 + r, out_dim - 1) * groups + (gg < groups ? gg : 0);
+            sraw[p] = S[at];
+            braw[p] = B[at];
         }
-        tot = group_sum<64>(tot);
-        if (lane == 0 && r < out_dim) sp.out[s][r] = tot;
-    };
-    // weights of rows i + 1 and i + 2 are in flight while row i is summed
-    mv_u32x4 w[3][NCH];
-    float sc[3][NCH], bi[3][NCH];
-    fetch(row0, w[0], sc[0], bi[0]);
-    fetch(row0 + 1, w[1], sc[1], bi[1]);
-    mv_static_for<ROWS>([&](auto it) __attribute__((always_inline)) {
-        constexpr int i = decltype(it)::value;
-        if (i + 2 < ROWS) fetch(row0 + i + 2, w[(i + 2) % 3], sc[(i + 2) % 3], bi[(i + 2) % 3]);
-        row(row0 + i, w[i % 3], sc[i % 3], bi[i % 3]);
-    });
+#pragma unroll
+        for (int i = tid; i < (128 * STEPS + 128) / 8; i += NTHR) *reinterpret_cast<mv_u32x4 *>(&zeros[8 * i]) = mv_u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int p = 0; p < XP; p++) {
+            const int r = tid + p * NTHR;
+            const bool live = 8 * r < in_dim;
+            const float4 a = xa[p], b = xb4[p];
+            float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            uint32_t hb[8], mb[8], lb[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {   // v = h + m + l, each a bf16 number (upper 16 bits)
+                if (!live) v[e] = 0.f;
+                hb[e] = __builtin_bit_cast(uint32_t, v[e]);
+                const float r1 = v[e] - __builtin_bit_cast(float, hb[e] & 0xffff0000u);
+                mb[e] = __builtin_bit_cast(uint32_t, r1);
+                lb[e] = __builtin_bit_cast(uint32_t, r1 - __builtin_bit_cast(float, mb[e] & 0xffff0000u));
+            }
+            const uint32_t hi16 = 0x07060302u;  // (upper half of the second operand, upper half of the first)
+            mv_u32x4 ph, pm, pl;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                ph[e] = __builtin_amdgcn_perm(hb[e + 4], hb[e], hi16);
+                pm[e] = __builtin_amdgcn_perm(mb[e + 4], mb[e], hi16);
+                pl[e] = __builtin_amdgcn_perm(lb[e + 4], lb[e], hi16);
+            }
+            *reinterpret_cast<mv_u32x4 *>(&xs[0][8 * r]) = ph;
+            *reinterpret_cast<mv_u32x4 *>(&xs[1][8 * r]) = pm;
+            *reinterpret_cast<mv_u32x4 *>(&xs[2][8 * r]) = pl;
+            float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+            sum = group_sum<8>(sum);
+            if ((tid & 7) == 0) xsum[r >> 3] = sum;
+        }
+#pragma unroll
+        for (int p = 0; p < SP; p++) {
+            const int i = tid + p * NTHR;
+            const int r = i / G, gg = i % G;
+            sc_l[gg][r] = gg < groups ? sraw[p] : (uint16_t)0;
+            bi_l[gg][r] = gg < groups ? braw[p] : (uint16_t)0;
+        }
+    }
+    __syncthreads();
+
+    // B operand: lane (column n, input octet g) reads part n % 3 of x if column n belongs to the
+    // scale group that octet g lies in (columns 0..2: octets 0, 1; columns 3..5: octets 2, 3), else zeros
+    const bool mine = n < 6 && (n / 3) == (g >> 1);
+    const uint16_t *xb = (mine ? &xs[n % 3][128 * STEPS * wave] : &zeros[0]) + 32 * g;
+    const int gsel = n >= 3 ? 1 : 0;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};   // rows 4g + i of the tile, this lane's column's share
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+        mv_f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t ww = w[st][j];
+            mv_u32x4 a;   // nibbles (0,4), (1,5), (2,6), (3,7) as bf16 pairs 1 + n/16
+            a[0] = ((ww << 3) & 0x00780078u) | 0x3F803F80u;
+            a[1] = ((ww >> 1) & 0x00780078u) | 0x3F803F80u;
+            a[2] = ((ww >> 5) & 0x00780078u) | 0x3F803F80u;
+            a[3] = ((ww >> 9) & 0x00780078u) | 0x3F803F80u;
+            const mv_bf16x8 b = *reinterpret_cast<const mv_bf16x8 *>(xb + 128 * st + 8 * j);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mv_bf16x8, a), b, d, 0, 0, 0);
+        }
+        // out += 16 s D: the scales of rows 4g .. 4g + 3 in this lane's group
+        const uint2 sb = *reinterpret_cast<const uint2 *>(&sc_l[2 * (wave * STEPS + st) + gsel][4 * g]);
+        acc[0] = fmaf(16.f * __builtin_bit_cast(float, sb.x << 16), d[0], acc[0]);
+        acc[1] = fmaf(16.f * __builtin_bit_cast(float, sb.x & 0xffff0000u), d[1], acc[1]);
+        acc[2] = fmaf(16.f * __builtin_bit_cast(float, sb.y << 16), d[2], acc[2]);
+        acc[3] = fmaf(16.f * __builtin_bit_cast(float, sb.y & 0xffff0000u), d[3], acc[3]);
+    }
+    {   // the X_g terms of this wave's 16 groups, one group per column lane
+        const int gg = 16 * wave + n;
+        const uint2 sb = *reinterpret_cast<const uint2 *>(&sc_l[gg][4 * g]);
+        const uint2 bb = *reinterpret_cast<const uint2 *>(&bi_l[gg][4 * g]);
+        const float xg = xsum[gg];
+        const float sv[4] = {__builtin_bit_cast(float, sb.x << 16), __builtin_bit_cast(float, sb.x & 0xffff0000u),
+                             __builtin_bit_cast(float, sb.y << 16), __builtin_bit_cast(float, sb.y & 0xffff0000u)};
+        const float bv[4] = {__builtin_bit_cast(float, bb.x << 16), __builtin_bit_cast(float, bb.x & 0xffff0000u),
+                             __builtin_bit_cast(float, bb.y << 16), __builtin_bit_cast(float, bb.y & 0xffff0000u)};
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] = fmaf(bv[i] - 16.f * sv[i], xg, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = group_sum<16>(acc[i]);
+    if (n == 0) *reinterpret_cast<mv_f32x4 *>(&red[wave][4 * g]) = mv_f32x4{acc[0], acc[1], acc[2], acc[3]};
+    __syncthreads();
+    if (tid < 16 && row0 + tid < out_dim) {
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) v += red[k][tid];
+        sp.out[s][row0 + tid] = v;
+    }
 }
 
 // Device pointers; one launch for up to 8 products (the reference batches a layer's
@@ -149,15 +215,16 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
         max_out = out_dim[i] > max_out ? out_dim[i] : max_out;
         max_in = in_dim[i] > max_in ? in_dim[i] : max_in;
     }
-    // rows per wave: as many as still leave every CU about two workgroups
-    const int rows = max_out >= 8 * 4 * 2 * num_cus ? 8 : max_out >= 4 * 4 * 2 * num_cus ? 4 : 2;
-    const dim3 grid((max_out + 4 * rows - 1) / (4 * rows), n);
-#define MFA_MV(NCH)                                                                                          \
-    if (rows == 8) hipLaunchKernelGGL((dequant_matvec_4bit_kernel<NCH, 8>), grid, dim3(256), 0, stream, sp);      \
-    else if (rows == 4) hipLaunchKernelGGL((dequant_matvec_4bit_kernel<NCH, 4>), grid, dim3(256), 0, stream, sp); \
-    else hipLaunchKernelGGL((dequant_matvec_4bit_kernel<NCH, 2>), grid, dim3(256), 0, stream, sp)
-    if (max_in <= 2048) { MFA_MV(1); } else if (max_in <= 4096) { MFA_MV(2); } else { MFA_MV(4); }
-#undef MFA_MV
+    MatvecTiles tl{};
+    for (int i = 0; i < n; i++) tl.first[i + 1] = tl.first[i] + (out_dim[i] + 15) / 16;
+    for (int i = n + 1; i <= kMvMaxSpecs; i++) tl.first[i] = tl.first[n];
+    const dim3 grid(tl.first[n]);
+    (void)max_out;
+    (void)num_cus;
+    if (max_in <= 1024) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<1>), grid, dim3(64), 0, stream, sp, tl, n);
+    else if (max_in <= 2048) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<2>), grid, dim3(128), 0, stream, sp, tl, n);
+    else if (max_in <= 4096) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<4>), grid, dim3(256), 0, stream, sp, tl, n);
+    else hipLaunchKernelGGL((dequant_matvec_mfma_kernel<8>), grid, dim3(512), 0, stream, sp, tl, n);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

@@ -42,6 +42,22 @@ def test_matvec_matches_oracle(mfa, oracle, out_dim, in_dim):
     assert rel_err(out, ref) <= TOL_F32
 
 
+@pytest.mark.parametrize("scale", [1e-30, 1e-6, 1e4, 1e30])
+def test_matvec_input_magnitudes(mfa, oracle, scale):
+    """The kernel splits x into three bf16 parts (exact for any f32 whose parts stay normal) and
+    converts the nibbles exactly: the result must not depend on the magnitude of x, nor on a
+    large common offset in x (group sums much larger than the signed part)."""
+    rng = np.random.default_rng(11)
+    out_dim, in_dim = 48, 2048
+    packed, sc, bi = _weights(rng, out_dim, in_dim, oracle)
+    x = (rng.standard_normal(in_dim) * scale).astype(np.float32)
+    ref = oracle.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, x)
+    assert rel_err(mfa.dequant_matvec_4bit_cpu(packed, sc, bi, in_dim, out_dim, x), ref) <= TOL_F32
+    xo = (x + np.float32(3.0 * scale)).astype(np.float32)
+    ref = oracle.dequant_matvec_4bit(packed, sc, bi, in_dim, out_dim, xo)
+    assert rel_err(mfa.dequant_matvec_4bit_cpu(packed, sc, bi, in_dim, out_dim, xo), ref) <= TOL_F32
+
+
 def test_batched_products_in_one_launch(mfa, oracle):
     """q, k and v projections of one layer as one call on device pointers
     (full_attn_forward.rs:193-227 batches them into one command buffer)."""
