@@ -298,7 +298,7 @@ def cpu_baseline(sample, Hq, Hkv, d, L, budget_s=12.0):
     t0 = time.perf_counter()
     ref = cref.sdpa(L, Hq, Hkv, d, q, g, kf, vf)
     first = time.perf_counter() - t0
-    n = int(max(1, min(20, budget_s / max(first, 1e-3))))
+    n = int(max(1, min(60, budget_s / max(first, 1e-3))))
     t0 = time.perf_counter()
     for _ in range(n):
         cref.sdpa(L, Hq, Hkv, d, q, g, kf, vf)
