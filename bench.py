@@ -478,6 +478,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
     ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
+    ap.add_argument("--f4-len", type=int, default=0, help="one cache length for --only f4 (default: 4096 and 32768)")
     ap.add_argument("--only", choices=["c4", "c5", "f3", "f4"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
@@ -496,7 +497,8 @@ def main():
         print(json.dumps({"f3_projection_matvecs": bench_matvec(a.steps, a.warmup, 0xC0FFEE + 6)}))
         return
     if a.only == "f4":
-        print(json.dumps({"f4_mla_folded_sdpa": bench_mla(a.steps, a.warmup, 0xC0FFEE + 7)}))
+        lens = (a.f4_len,) if a.f4_len else (4096, 32768)
+        print(json.dumps({"f4_mla_folded_sdpa": bench_mla(a.steps, a.warmup, 0xC0FFEE + 7, lens)}))
         return
     if a.only == "c5":
         print(json.dumps({"c5_token_sweep_48_layers": bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)}))

@@ -93,7 +93,8 @@ int mfa_set_linear_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *conv_w_b
                            const float *a_log, const uint16_t *dt_bias_bf16,
                            const uint16_t *norm_w_bf16);
 
-/* Override the split-K partition count of the decode kernel (0 = automatic).
+/* Override the split-K partition count of the decode kernel and of
+ * mfa_mla_sdpa_folded_dev (0 = automatic).
  * The result must not depend on it; tests use it to check exactly that, as
  * the reference checks tiled against single-shot MLA (tests/mla_sdpa_tiled.rs:
  * 176-216). */

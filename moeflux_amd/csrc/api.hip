@@ -800,7 +800,7 @@ int mfa_mla_sdpa_folded_dev(mfa_ctx *ctx, int32_t num_heads, int32_t kv_lora_ran
     if (!c || !q_prime || !q_pe || !latent_cache || !rope_k_cache || !v_combine)
         return fail(MFA_ERR_INVALID, "NULL argument");
     MFA_TRY(mla_check(num_heads, kv_lora_rank, qk_rope_head_dim, cache_len));
-    const MlaPlan plan = mla_plan(num_heads, cache_len, c->num_cus);
+    const MlaPlan plan = mla_plan(num_heads, cache_len, c->num_cus, c->forced_splits);
     MFA_TRY(ensure_workspace_elems(c, mla_workspace_o_elems(plan, kv_lora_rank), mla_workspace_ml_elems(plan)));
     return launch_mla_sdpa_folded(c->stream, num_heads, kv_lora_rank, qk_rope_head_dim, cache_len, softmax_scale,
                                   q_prime, q_pe, latent_cache, rope_k_cache, v_combine, workspace(c), plan);

@@ -198,7 +198,7 @@ struct MlaPlan {
     int nwg_heads;  // workgroups along the heads (4 groups each)
 };
 bool mla_shape_supported(int kv_lora_rank, int qk_rope_head_dim);
-MlaPlan mla_plan(int H, int L, int num_cus);
+MlaPlan mla_plan(int H, int L, int num_cus, int forced_splits = 0);
 size_t mla_workspace_o_elems(const MlaPlan &p, int R);
 size_t mla_workspace_ml_elems(const MlaPlan &p);
 int launch_mla_sdpa_folded(hipStream_t stream, int H, int R, int P, int L, float softmax_scale,

@@ -89,6 +89,28 @@ def test_mla_device_entry_reuses_the_workspace(mfa, oracle):
             assert rel_err(do.to_host(), oracle.mla_sdpa_folded(H, R, P, L, 0.07, qp, qe, lat, rk)) <= TOL_F32
 
 
+def test_mla_split_count_invariance(mfa, oracle):
+    """tests/mla_sdpa_tiled.rs:143-185 compares the tiled kernel with the single-pass one; here the
+    number of partitions of the cache is forced to 1, 3, 16 and 64 and every result is held to
+    the oracle."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    H, L = 48, 1500
+    qp, qe, lat, rk = _random(21, H, L)
+    ref = oracle.mla_sdpa_folded(H, R, P, L, 0.09, qp, qe, lat, rk)
+    d = [DeviceArray.from_host(a) for a in (qp, qe, lat, rk)]
+    do = DeviceArray((H * R,), np.float32, zero=True)
+    with mfa.Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64,
+                        kv_capacity=4)) as c:
+        for splits in (1, 3, 16, 64):
+            assert c.lib.mfa_set_num_splits(c.h, splits) == 0
+            rc = c.lib.mfa_mla_sdpa_folded_dev(c.h, H, R, P, L, C.c_float(0.09), d[0].ptr, d[1].ptr, d[2].ptr,
+                                               d[3].ptr, do.ptr)
+            assert rc == 0, ffi.last_error()
+            c.sync()
+            assert rel_err(do.to_host(), ref) <= TOL_F32, splits
+
+
 def test_mla_size_independent_properties(mfa):
     """At the full length (32768 positions, 128 heads), where the oracle would take minutes:
     a zero query gives the mean latent row; equal latent rows come back whatever the weights;
