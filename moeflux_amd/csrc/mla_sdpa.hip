@@ -30,8 +30,8 @@
 //     ends up with channel j at four positions).  The value product's 32 slots are the hi
 //     parts of the 16 positions followed by their lo parts, so that with P = [p_hi | p_hi]
 //     one instruction adds x_hi p_hi + x_lo p_hi and a second with [p_lo | 0] adds x_hi p_lo.
-//     The value waves fetch and split the latent rows (two channels x 16 positions per
-//     thread), the score waves the rotary keys.
+//     The value waves fetch and split 12 of a block's 16 latent rows (two channels per
+//     thread), the score waves the other 4 and the rotary keys, which evens out the two roles.
 //     Partials (unnormalised O, running max and sum per head) go to the workspace in the
 //     layout of the decode kernel's partials, and sdpa_merge_kernel combines them.
 #include "sdpa_wave.h"
@@ -67,6 +67,7 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
     static_assert(NROLE == 256 && R == 512 && P == 64, "the staging maps 256 threads per role onto a 16 x (512 + 64) block");
     constexpr int KPLANE = kMlaBlk * KROW * 2;           // bytes of one plane (hi or lo) of a block
     constexpr int KBUF = 2 * KPLANE;                     // one buffer
+    constexpr int VPOS = 12;              // positions of a block whose latent rows the value waves stage; the score waves take the rest
     __shared__ __attribute__((aligned(16))) unsigned char smem[3 * KBUF];
     __shared__ __attribute__((aligned(16))) uint16_t pbuf[2][HG][2][16][kMlaBlk];  // weights [buffer][group][hi|lo][head][position]
     __shared__ float abuf[2][HG][16];                                             // rescale factor of a block, per head
@@ -97,13 +98,16 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
 
     if (score_role) {
         // ================= scores and softmax of head group hgl =================
-        // staging: the rotary keys, two channels at positions rp and rp + 8
+        // staging: the rotary keys, two channels at positions rp and rp + 8, and the latent rows the value waves leave
         const int rp = rtid >> 5, rc2 = rtid & 31;
-        f32x2 rraw[2];
+        f32x2 rraw[2], lraw[kMlaBlk - VPOS];
         auto fetch =[&](int b) {
 #pragma unroll
             for (int k = 0; k < 2; k++)
                 rraw[k] = mla_load2(rope_k + (size_t)min(clampb(b) * kMlaBlk + rp + 8 * k, L - 1) * P + 2 * rc2);
+#pragma unroll
+            for (int j = VPOS; j < kMlaBlk; j++)
+                lraw[j - VPOS] = mla_load2(latent + (size_t)min(clampb(b) * kMlaBlk + j, L - 1) * R + 2 * rtid);
         };
         const int kr_off = (rp * KROW + R + 2 * rc2) * 2;
         auto commit =[&](int b) {
@@ -114,6 +118,13 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
                 split_pair(rraw[k][0], rraw[k][1], rh, rl);
                 *reinterpret_cast<uint32_t *>(base + kr_off + 8 * k * KROW * 2) = rh;
                 *reinterpret_cast<uint32_t *>(base + kr_off + 8 * k * KROW * 2 + KPLANE) = rl;
+            }
+#pragma unroll
+            for (int j = VPOS; j < kMlaBlk; j++) {   // the last latent rows of the block, channels 2 rtid, 2 rtid + 1
+                uint32_t hi, lo;
+                split_pair(lraw[j - VPOS][0], lraw[j - VPOS][1], hi, lo);
+                *reinterpret_cast<uint32_t *>(base + 4 * rtid + j * KROW * 2) = hi;
+                *reinterpret_cast<uint32_t *>(base + 4 * rtid + j * KROW * 2 + KPLANE) = lo;
             }
         };
         fetch(b0);
@@ -196,18 +207,18 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
         __syncthreads();  // iteration b1 - 1: the value waves accumulate the last block
     } else {
         // ================= values of head group hgl =================
-        // staging: the latent rows, channels 2 c2, 2 c2 + 1 at the block's 16 positions
+        // staging: the latent rows, channels 2 c2, 2 c2 + 1 at the block's first VPOS positions
         const int c2 = rtid;
-        f32x2 raw[16];
+        f32x2 raw[VPOS];
         auto fetch =[&](int b) {
 #pragma unroll
-            for (int j = 0; j < 16; j++)
+            for (int j = 0; j < VPOS; j++)
                 raw[j] = mla_load2(latent + (size_t)min(clampb(b) * kMlaBlk + j, L - 1) * R + 2 * c2);
         };
         auto commit =[&](int b) {
             unsigned char *base = bufof(b) + 4 * c2;
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
+            for (int j = 0; j < VPOS; j++) {
                 uint32_t hi, lo;
                 split_pair(raw[j][0], raw[j][1], hi, lo);
                 *reinterpret_cast<uint32_t *>(base + j * KROW * 2) = hi;
