@@ -29,7 +29,8 @@
 //     j/4 + 12; with lane L pointing at position L/4, channels 4 (L % 4) .. + 3, lane j
 //     ends up with channel j at four positions).  The value product's 32 slots are the hi
 //     parts of the 16 positions followed by their lo parts, so that with P = [p_hi | p_hi]
-//     one instruction adds x_hi p_hi + x_lo p_hi and a second with [p_lo | 0] adds x_hi p_lo.
+//     one instruction adds x_hi p_hi + x_lo p_hi and a second with [p_lo | p_lo] adds x_hi p_lo
+//     (and x_lo p_lo, which comes for free).
 //     The value waves fetch and split 12 of a block's 16 latent rows (two channels per
 //     thread), the score waves the other 4 and the rotary keys, which evens out the two roles.
 //     Partials (unnormalised O, running max and sum per head) go to the workspace in the
@@ -247,8 +248,7 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
             const unsigned char *base = bufof(it) + tr_rd;
             // lane (n, g): weights of head n at positions 8 (g & 1) .. + 7
             const bf16x8 pb_h = mla_lds8(&pbuf[it & 1][hgl][0][n][8 * (g & 1)]);
-            bf16x8 pb_l = mla_lds8(&pbuf[it & 1][hgl][1][n][8 * (g & 1)]);
-            if (!hi_slots) pb_l = as_bf16x8(uint4{0u, 0u, 0u, 0u});  // no x_lo p_lo term
+            const bf16x8 pb_l = mla_lds8(&pbuf[it & 1][hgl][1][n][8 * (g & 1)]);
             const float alpha = abuf[it & 1][hgl][n];
             if (__any(alpha != 1.f)) {
 #pragma unroll
