@@ -87,6 +87,33 @@ def test_batched_products_in_one_launch(mfa, oracle):
             assert rel_err(o.to_host(), r) <= TOL_F32
 
 
+def test_batched_products_of_different_widths(mfa, oracle):
+    """Eight products in one launch whose input widths differ (the launch is shaped by the widest)
+    and whose row counts do not fill their last 16-row tile."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    rng = np.random.default_rng(8)
+    shapes = [(100, 4096), (33, 64), (512, 2048), (1, 1024), (17, 4160), (64, 192), (250, 3072), (16, 8192)]
+    keep, refs, outs = [], [], []
+    specs = (ffi.mfa_matvec_spec * len(shapes))()
+    for i, (od, idim) in enumerate(shapes):
+        packed, sc, bi = _weights(rng, od, idim, oracle)
+        x = rng.standard_normal(idim).astype(np.float32)
+        refs.append(oracle.dequant_matvec_4bit(packed, sc, bi, idim, od, x))
+        dw, ds, db, dx = (DeviceArray.from_host(a) for a in (packed, sc, bi, x))
+        do = DeviceArray((od,), np.float32, zero=True)
+        keep += [dw, ds, db, dx]
+        outs.append(do)
+        specs[i] = ffi.mfa_matvec_spec(dw.ptr, ds.ptr, db.ptr, dx.ptr, do.ptr, od, idim)
+    with mfa.Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64,
+                        kv_capacity=4)) as c:
+        rc = c.lib.mfa_dequant_matvec_4bit_dev(c.h, len(shapes), C.byref(specs))
+        assert rc == 0, ffi.last_error()
+        c.sync()
+        for o, r, sh in zip(outs, refs, shapes):
+            assert rel_err(o.to_host(), r) <= TOL_F32, sh
+
+
 def test_matvec_errors(mfa):
     """cpu_matvec.rs:92-97: in_dim must be a multiple of the group size; NULL and shape checks."""
     from moeflux_amd import ffi
