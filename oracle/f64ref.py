@@ -167,3 +167,22 @@ def attn_prologue(pos, Hq, Hkv, d, rotary_dim, theta, eps, q_norm_bf16, k_norm_b
     k = rotary(pos, Hkv, d, rotary_dim, theta, rms_norm_per_head(Hkv, d, eps, k_norm_bf16, k_in))
     return q, qp[:, 1].reshape(-1).copy(), k, np.asarray(v_in, np.float64).copy()
 
+
+def mla_sdpa_folded(H, R, P, L, scale, q_prime, q_pe, latent, rope_k):
+    """Attention over a latent cache: scores over [latent | rope_k], softmax, weighted sum of latent."""
+    qp = np.asarray(q_prime, np.float64).reshape(H, R)
+    qe = np.asarray(q_pe, np.float64).reshape(H, P)
+    lat = np.asarray(latent, np.float64).reshape(L, R)
+    rk = np.asarray(rope_k, np.float64).reshape(L, P)
+    s = (np.einsum("hr,lr->hl", qp, lat) + np.einsum("hp,lp->hl", qe, rk)) * scale
+    return np.einsum("hl,lr->hr", softmax(s, axis=1), lat)
+
+
+def dequant_matvec_4bit(packed, scales_bf16, biases_bf16, in_dim, out_dim, x):
+    """Group-64 affine 4-bit weights: nibble n of word w of a row is input 8 w + n."""
+    pk = np.asarray(packed, np.uint32).reshape(out_dim, in_dim // 8)
+    nib = np.stack([(pk >> (4 * n)) & 0xF for n in range(8)], axis=-1).reshape(out_dim, in_dim).astype(np.float64)
+    sc = np.repeat(bf16_bits_to_f64(scales_bf16).reshape(out_dim, in_dim // 64), 64, axis=1)
+    bi = np.repeat(bf16_bits_to_f64(biases_bf16).reshape(out_dim, in_dim // 64), 64, axis=1)
+    return (nib * sc + bi) @ np.asarray(x, np.float64)
+

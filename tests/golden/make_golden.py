@@ -1,5 +1,5 @@
-"""Writes tests/golden/attention_f64.json and tests/golden/attn_prologue_f64.json: small cases of every function on the
-attention path, inputs and float64 expected outputs.
+"""Writes tests/golden/attention_f64.json, attn_prologue_f64.json and around_the_core_f64.json: small cases of every
+function on the attention path and around it, inputs and float64 expected outputs.
 
 The expected values come from oracle/f64ref.py — vectorised float64 numpy built
 on library routines (einsum, scipy.special.softmax / expit), written from the
@@ -47,8 +47,31 @@ def prologue_cases():
         json.dump({"attn_prologue": cases}, f)
 
 
+def around_the_core_cases():
+    """Attention over a latent cache and the 4-bit dequantising matrix-vector product."""
+    rng = np.random.default_rng(20261127)
+    mla, mv = [], []
+    for (H, R, P, L, scale) in [(2, 8, 4, 1, 0.5), (3, 16, 4, 9, 0.29), (5, 32, 8, 40, 0.16), (16, 64, 16, 33, 0.11)]:
+        qp, qe = r32(rng, H, R, scale=0.4), r32(rng, H, P, scale=0.4)
+        lat, rk = r32(rng, L, R), r32(rng, L, P)
+        out = f64ref.mla_sdpa_folded(H, R, P, L, scale, qp, qe, lat, rk)
+        mla.append(dict(H=H, R=R, P=P, L=L, scale=scale, q_prime=lst(qp), q_pe=lst(qe), latent=lst(lat),
+                        rope_k=lst(rk), out=lst(out)))
+    for (od, idim) in [(1, 64), (3, 128), (7, 320), (16, 512)]:
+        packed = rng.integers(0, 2 ** 32, size=(od, idim // 8), dtype=np.uint64).astype(np.uint32)
+        sc = cref.f32_to_bf16(np.abs(rng.standard_normal((od, idim // 64))) * 0.02 + 0.003)
+        bi = cref.f32_to_bf16(rng.standard_normal((od, idim // 64)) * 0.1)
+        x = r32(rng, idim)
+        out = f64ref.dequant_matvec_4bit(packed, sc, bi, idim, od, x)
+        mv.append(dict(out_dim=od, in_dim=idim, packed=lst(packed), scales=lst(sc), biases=lst(bi), x=lst(x),
+                       out=lst(out)))
+    with open(os.path.join(HERE, "around_the_core_f64.json"), "w") as f:
+        json.dump({"mla_sdpa_folded": mla, "dequant_matvec_4bit": mv}, f)
+
+
 def main():
     prologue_cases()
+    around_the_core_cases()
     rng = np.random.default_rng(20261125)
     cases = {"sdpa": [], "gdn_step": [], "conv1d": [], "rms_norm_qk": [], "decay_beta": [],
              "delta_net_step": [], "rms_norm_gated": [], "prefill_attn": []}

@@ -464,3 +464,29 @@ def test_mla_closed_forms():
     rk2[5] = 60.0 * qe[1] / np.dot(qe[1], qe[1])
     out = f(qp * 0, qe, lat, rk2)
     assert np.allclose(out[1], lat[5], rtol=1e-4, atol=1e-5)
+
+
+# ---- committed float64 fixtures for the functions around the core --------------------
+
+ATC = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "around_the_core_f64.json")))
+
+
+@pytest.mark.parametrize("case", ATC["mla_sdpa_folded"], ids=lambda c: f"H{c['H']}_L{c['L']}")
+def test_mla_golden(case):
+    c = case
+    got = cref.mla_sdpa_folded(c["H"], c["R"], c["P"], c["L"], c["scale"], np.array(c["q_prime"], np.float32),
+                               np.array(c["q_pe"], np.float32), np.array(c["latent"], np.float32),
+                               np.array(c["rope_k"], np.float32))
+    assert rel_err(got, np.array(c["out"])) <= F32
+
+
+@pytest.mark.parametrize("case", ATC["dequant_matvec_4bit"], ids=lambda c: f"{c['out_dim']}x{c['in_dim']}")
+def test_dequant_matvec_golden(case):
+    c = case
+    got = cref.dequant_matvec_4bit(np.array(c["packed"], np.uint32), np.array(c["scales"], np.uint16),
+                                   np.array(c["biases"], np.uint16), c["in_dim"], c["out_dim"],
+                                   np.array(c["x"], np.float32))
+    # a row is a signed sum of in_dim terms accumulated in f32, as the reference accumulates it: the
+    # rounding of the partial sums is relative to their size, not to the (cancelled) result
+    assert rel_err(got, np.array(c["out"])) <= 1e-5
+
