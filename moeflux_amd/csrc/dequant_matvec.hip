@@ -12,16 +12,14 @@
 //   * A nibble n becomes the bf16 number 1 + n/16 (exponent bits of 1.0, n in the top four
 //     mantissa bits): two nibbles per shift + and-or, exact, one instruction per weight.
 //   * x is split into three bf16 parts by truncation (x = h + m + l exactly), which sit in
-//     three columns of the B operand; a 16x16x32 instruction therefore gives, per row,
+//     three rows of the other operand; a 16x16x32 instruction therefore gives, per row of W,
 //     sum (1 + n/16) x exactly up to f32 accumulation.
 //   * One instruction covers 32 inputs per lane group, i.e. two scale groups of 64 per four
-//     instructions: columns 0..2 carry the first group's x (zero elsewhere), columns 3..5 the
+//     instructions: operand rows 0..2 carry the first group's x (zero elsewhere), rows 4..6 the
 //     second's, so the two groups' sums stay apart in one accumulator tile.
 //   * Per group g and row r:  out += 16 s (D - X_g) + b X_g  with X_g = sum x over the group;
 //     D is about 1.5 X_g, so the subtraction costs no more than two bits.
-// A workgroup owns 16 rows (the M side of the tile); its waves split the inputs in runs of
-// 1024, each lane requesting its 8 x 16 bytes of weights before anything else, and x, the
-// scales and the biases are staged in LDS while those requests are in flight.
+#include <cstdint>
 #include <type_traits>
 
 #include "gdn_device.h"
@@ -49,152 +47,227 @@ struct MatvecTiles {
     int first[kMvMaxSpecs + 1];  // first 16-row tile of every product, and the total
 };
 
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void dequant_matvec_mfma_kernel(MatvecSpecs sp, MatvecTiles tl, int n_specs) {
-    constexpr int NTHR = WAVES * 64;
+// Eight consecutive bf16 scales (or biases) of one row, groups first .. first + 7, as stored.
+// ALIGNED: every row starts on a 16-byte boundary and has a multiple of 8 groups.
+template <bool ALIGNED>
+__device__ inline mv_u32x4 load_sb8(const uint16_t *row, int first, int groups) {
+    if constexpr (ALIGNED) return *reinterpret_cast<const mv_u32x4 *>(row + (first < groups ? first : 0));
+    uint32_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) e[i] = first + i < groups ? row[first + i] : 0u;
+    return mv_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+}
+
+// The product a tile belongs to, found and read with compile-time indices only (the tables
+// stay in scalar registers; an index computed at run time would be looked up lane by lane).
+struct Product {
+    const uint32_t *w;
+    const uint16_t *scales, *biases;
+    const float *x;
+    float *out;
+    int out_dim, in_dim, first;
+};
+__device__ inline Product mv_product_of(const MatvecSpecs &sp, const MatvecTiles &tl, int t) {
+    int s = 0;   // first[] does not decrease and is padded with the total
+#pragma unroll
+    for (int i = 1; i < kMvMaxSpecs; i++) s += t >= tl.first[i] ? 1 : 0;
+    s = __builtin_amdgcn_readfirstlane(s);
+    Product q;
+    q.w = sp.w[0]; q.scales = sp.scales[0]; q.biases = sp.biases[0]; q.x = sp.x[0]; q.out = sp.out[0];
+    q.out_dim = sp.out_dim[0]; q.in_dim = sp.in_dim[0]; q.first = tl.first[0];
+#pragma unroll
+    for (int i = 1; i < kMvMaxSpecs; i++) {
+        const bool hit = s == i;
+        q.w = hit ? sp.w[i] : q.w;
+        q.scales = hit ? sp.scales[i] : q.scales;
+        q.biases = hit ? sp.biases[i] : q.biases;
+        q.x = hit ? sp.x[i] : q.x;
+        q.out = hit ? sp.out[i] : q.out;
+        q.out_dim = hit ? sp.out_dim[i] : q.out_dim;
+        q.in_dim = hit ? sp.in_dim[i] : q.in_dim;
+        q.first = hit ? tl.first[i] : q.first;
+    }
+    return q;
+}
+
+// One workgroup per TILES tiles of 16 rows (TILES = 1 is what is launched: with two, x is read
+// and split half as often, but fewer waves fit a CU and the launch as a whole was slower); its
+// waves split the inputs in runs of 1024, and each wave stages the part of x it uses itself.
+//
+// The weights are the B side of the matrix instruction (column = row of the tile) and the
+// parts of x the A side: row 0..2 of A are the three parts of x restricted to the first scale
+// group of a 128-input step, rows 4..6 the same for the second group.  Lane (n, g) of the
+// result then holds, for g = 0 and g = 1, the three partial sums of row n of the tile over
+// scale group g of the step - and needs only its own row's scale to finish it.  Lanes
+// (n, 2) and (n, 3), whose results are zero, add the bias terms b X_g of the even and odd groups.
+//
+// Loads come back in the order they were asked for, so the order of the requests is the order
+// of use: x (staged in LDS while everything else is on its way), the row's scales and biases
+// (16 bytes per lane straight into registers), then the 8 x 16 bytes of weights per lane.
+template <int WAVES, bool SB16, int TILES>
+__device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const MatvecTiles &tl) {
     constexpr int KP = WAVES * 1024;   // inputs covered by the workgroup (in_dim padded)
     constexpr int G = KP / 64;         // scale groups
     constexpr int STEPS = 8;           // 128-input steps per wave
     __shared__ __attribute__((aligned(16))) uint16_t xs[3][KP];       // bf16 parts of x; within a run of 8 inputs the order is 0,4,1,5,2,6,3,7
-    __shared__ __attribute__((aligned(16))) uint16_t zeros[128 * STEPS + 128];  // what the other lanes of the B operand read
-    // scales and biases of the tile's rows as stored (bf16), [group][row]; + 4: the staging writes walk the groups
-    __shared__ __attribute__((aligned(8))) uint16_t sc_l[G][16 + 4], bi_l[G][16 + 4];
+    __shared__ __attribute__((aligned(16))) uint16_t zeros[128 * STEPS + 128];  // what the other lanes of the A operand read
     __shared__ float xsum[G];
-    __shared__ __attribute__((aligned(16))) float red[WAVES][16];
+    __shared__ float red[WAVES][16 * TILES];
 
-    int s = 0;
-    while (s + 1 < n_specs && (int)blockIdx.x >= tl.first[s + 1]) s++;
-    const int row0 = ((int)blockIdx.x - tl.first[s]) * 16;
-    const int in_dim = sp.in_dim[s], out_dim = sp.out_dim[s];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const int nchunk = in_dim >> 5, groups = in_dim >> 6, words = in_dim >> 3;
+    const int t = blockIdx.x;
+    const Product q = mv_product_of(sp, tl, t);
 
-    // ---- weights: row n of the tile, 32-input chunk 4 S + g of step S; all requested now ----
-    mv_u32x4 w[STEPS];
-    {
-        const uint32_t *wrow = sp.w[s] + (size_t)min(row0 + n, out_dim - 1) * words;
+    mv_u32x4 w[TILES][STEPS];   // row n of tile T, 32-input chunk 4 S + g of step S
+    mv_u32x4 q0[TILES], q1[TILES];   // groups 16 wave .. + 15 of that row: scales in lanes g < 2, biases in the others
+    auto fetch = [&]() __attribute__((always_inline)) {
+        const int in_dim = q.in_dim, out_dim = q.out_dim;
+        const int nchunk = in_dim >> 5, groups = in_dim >> 6, words = in_dim >> 3;
+        // the scales before the weights: the first step of the product needs them, and loads
+        // come back in the order they were asked for
+#pragma unroll
+        for (int T = 0; T < TILES; T++) {
+            const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
+            const uint16_t *sb = (g < 2 ? q.scales : q.biases) + (size_t)row * groups;
+            q0[T] = load_sb8<SB16>(sb, 16 * wave, groups);
+            q1[T] = load_sb8<SB16>(sb, 16 * wave + 8, groups);
+        }
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
             const int c = 4 * (wave * STEPS + st) + g;
-            w[st] = *reinterpret_cast<const mv_u32x4 *>(wrow + (c < nchunk ? c : 0) * 4);  // past the row: any chunk, x is 0 there
+#pragma unroll
+            for (int T = 0; T < TILES; T++) {
+                const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
+                w[T][st] = *reinterpret_cast<const mv_u32x4 *>(q.w + (size_t)row * words + (c < nchunk ? c : 0) * 4);  // past the row: any chunk, x is 0 there
+            }
         }
-    }
-    // ---- stage x (a run of 8 inputs per thread and pass), the scales and the biases; every
-    //      request first, so that the workgroup pays one round trip, not one per pass ----
-    {
-        constexpr int XP = KP / 8 / NTHR;       // passes over x
-        constexpr int SP = 16 * G / NTHR;   // passes over the (row, group) pairs
-        const float *x = sp.x[s];
-        const uint16_t *S = sp.scales[s], *B = sp.biases[s];
-        float4 xa[XP], xb4[XP];
-        uint16_t sraw[SP], braw[SP];
+    };
+    // x of product s: three bf16 parts by truncation (x = h + m + l exactly) and the group sums
+    constexpr int XP = 2;       // passes, a run of 8 inputs per lane and pass
+    float4 xa[XP], xb4[XP];
+    auto request_x = [&]() __attribute__((always_inline)) {
+        const float *x = q.x;
+        const int in_dim = q.in_dim;
 #pragma unroll
         for (int p = 0; p < XP; p++) {
-            const int r = tid + p * NTHR;
+            const int r = 128 * wave + lane + 64 * p;   // a wave stages the 1024 inputs it will use itself
             const int at = 8 * r < in_dim ? 8 * r : 0;
             xa[p] = load_f4(x + at);
             xb4[p] = load_f4(x + at + 4);
         }
-#pragma unroll
-        for (int p = 0; p < SP; p++) {
-            const int i = tid + p * NTHR;
-            const int r = i / G, gg = i % G;
-            const size_t at = (size_t)min(row0 + r, out_dim - 1) * groups + (gg < groups ? gg : 0);
-            sraw[p] = S[at];
-            braw[p] = B[at];
-        }
-#pragma unroll
-        for (int i = tid; i < (128 * STEPS + 128) / 8; i += NTHR) *reinterpret_cast<mv_u32x4 *>(&zeros[8 * i]) = mv_u32x4{0u, 0u, 0u, 0u};
+    };
+    auto stage_x = [&]() __attribute__((always_inline)) {
+        const int in_dim = q.in_dim;
 #pragma unroll
         for (int p = 0; p < XP; p++) {
-            const int r = tid + p * NTHR;
-            const bool live = 8 * r < in_dim;
-            const float4 a = xa[p], b = xb4[p];
-            float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-            uint32_t hb[8], mb[8], lb[8];
+            const int r = 128 * wave + lane + 64 * p;   // a wave stages the 1024 inputs it will use itself
+            mv_u32x4 ph = {0u, 0u, 0u, 0u}, pm = ph, pl = ph;
+            float sum = 0.f;
+            if (8 * r < in_dim) {   // past the end of x: zeros
+                const float4 a = xa[p], b = xb4[p];
+                const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+                uint32_t hb[8], mb[8], lb[8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {   // v = h + m + l, each a bf16 number (upper 16 bits)
-                if (!live) v[e] = 0.f;
-                hb[e] = __builtin_bit_cast(uint32_t, v[e]);
-                const float r1 = v[e] - __builtin_bit_cast(float, hb[e] & 0xffff0000u);
-                mb[e] = __builtin_bit_cast(uint32_t, r1);
-                lb[e] = __builtin_bit_cast(uint32_t, r1 - __builtin_bit_cast(float, mb[e] & 0xffff0000u));
-            }
-            const uint32_t hi16 = 0x07060302u;  // (upper half of the second operand, upper half of the first)
-            mv_u32x4 ph, pm, pl;
+                for (int e = 0; e < 8; e++) {   // v = h + m + l, each a bf16 number (upper 16 bits)
+                    hb[e] = __builtin_bit_cast(uint32_t, v[e]);
+                    const float r1 = v[e] - __builtin_bit_cast(float, hb[e] & 0xffff0000u);
+                    mb[e] = __builtin_bit_cast(uint32_t, r1);
+                    lb[e] = __builtin_bit_cast(uint32_t, r1 - __builtin_bit_cast(float, mb[e] & 0xffff0000u));
+                }
+                const uint32_t hi16 = 0x07060302u;  // (upper half of the second operand, upper half of the first)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                ph[e] = __builtin_amdgcn_perm(hb[e + 4], hb[e], hi16);
-                pm[e] = __builtin_amdgcn_perm(mb[e + 4], mb[e], hi16);
-                pl[e] = __builtin_amdgcn_perm(lb[e + 4], lb[e], hi16);
+                for (int e = 0; e < 4; e++) {
+                    ph[e] = __builtin_amdgcn_perm(hb[e + 4], hb[e], hi16);
+                    pm[e] = __builtin_amdgcn_perm(mb[e + 4], mb[e], hi16);
+                    pl[e] = __builtin_amdgcn_perm(lb[e + 4], lb[e], hi16);
+                }
+                sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
             }
             *reinterpret_cast<mv_u32x4 *>(&xs[0][8 * r]) = ph;
             *reinterpret_cast<mv_u32x4 *>(&xs[1][8 * r]) = pm;
             *reinterpret_cast<mv_u32x4 *>(&xs[2][8 * r]) = pl;
-            float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
             sum = group_sum<8>(sum);
             if ((tid & 7) == 0) xsum[r >> 3] = sum;
         }
-#pragma unroll
-        for (int p = 0; p < SP; p++) {
-            const int i = tid + p * NTHR;
-            const int r = i / G, gg = i % G;
-            sc_l[gg][r] = gg < groups ? sraw[p] : (uint16_t)0;
-            bi_l[gg][r] = gg < groups ? braw[p] : (uint16_t)0;
-        }
-    }
-    __syncthreads();
+    };
 
-    // B operand: lane (column n, input octet g) reads part n % 3 of x if column n belongs to the
-    // scale group that octet g lies in (columns 0..2: octets 0, 1; columns 3..5: octets 2, 3), else zeros
-    const bool mine = n < 6 && (n / 3) == (g >> 1);
-    const uint16_t *xb = (mine ? &xs[n % 3][128 * STEPS * wave] : &zeros[0]) + 32 * g;
-    const int gsel = n >= 3 ? 1 : 0;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};   // rows 4g + i of the tile, this lane's column's share
+    // A operand: lane (part row n, input octet g) reads part n % 4 of x if row n belongs to the
+    // scale group that octet g lies in (rows 0..2: octets 0, 1; rows 4..6: octets 2, 3), else zeros
+    const bool mine = n < 8 && (n & 3) < 3 && (n >> 2) == (g >> 1);
+    const uint16_t *xb = (mine ? &xs[n & 3][128 * STEPS * wave] : &zeros[0]) + 32 * g;
+    const int half = g & 1, sh = half ? 0 : 16;
+    const float *xs_g = &xsum[16 * wave + half];
+    request_x();
+    fetch();
+    // (every wave writes all of the zeros: no wave then has to wait for another before its product)
+#pragma unroll
+    for (int i = lane; i < (128 * STEPS + 128) / 8; i += 64) *reinterpret_cast<mv_u32x4 *>(&zeros[8 * i]) = mv_u32x4{0u, 0u, 0u, 0u};
+    stage_x();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // (x & mask) | bits in one instruction; it takes one constant from a scalar register and one
+    // from a vector register, which the compiler will not arrange by itself for two literals
+    uint32_t nib_mask = 0x00780078u, one_one = 0x3F803F80u;
+    asm volatile("" : "+s"(nib_mask), "+v"(one_one));
+    auto and_or = [](uint32_t x, uint32_t mask, uint32_t bits) __attribute__((always_inline)) {
+        uint32_t r;
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(bits));
+        return r;
+    };
+    float acc[TILES];
+#pragma unroll
+    for (int T = 0; T < TILES; T++) acc[T] = 0.f;
 #pragma unroll
     for (int st = 0; st < STEPS; st++) {
-        mv_f32x4 d = {0.f, 0.f, 0.f, 0.f};
+        mv_f32x4 d[TILES];
+#pragma unroll
+        for (int T = 0; T < TILES; T++) d[T] = mv_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t ww = w[st][j];
-            mv_u32x4 a;   // nibbles (0,4), (1,5), (2,6), (3,7) as bf16 pairs 1 + n/16
-            a[0] = ((ww << 3) & 0x00780078u) | 0x3F803F80u;
-            a[1] = ((ww >> 1) & 0x00780078u) | 0x3F803F80u;
-            a[2] = ((ww >> 5) & 0x00780078u) | 0x3F803F80u;
-            a[3] = ((ww >> 9) & 0x00780078u) | 0x3F803F80u;
             const mv_bf16x8 b = *reinterpret_cast<const mv_bf16x8 *>(xb + 128 * st + 8 * j);
-            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mv_bf16x8, a), b, d, 0, 0, 0);
+#pragma unroll
+            for (int T = 0; T < TILES; T++) {
+                const uint32_t ww = w[T][st][j];
+                mv_u32x4 a;   // nibbles (0,4), (1,5), (2,6), (3,7) as bf16 pairs 1 + n/16
+                a[0] = and_or(ww << 3, nib_mask, one_one);
+                a[1] = and_or(ww >> 1, nib_mask, one_one);
+                a[2] = and_or(ww >> 5, nib_mask, one_one);
+                a[3] = and_or(ww >> 9, nib_mask, one_one);
+                d[T] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, __builtin_bit_cast(mv_bf16x8, a), d[T], 0, 0, 0);
+            }
         }
-        // out += 16 s D: the scales of rows 4g .. 4g + 3 in this lane's group
-        const uint2 sb = *reinterpret_cast<const uint2 *>(&sc_l[2 * (wave * STEPS + st) + gsel][4 * g]);
-        acc[0] = fmaf(16.f * __builtin_bit_cast(float, sb.x << 16), d[0], acc[0]);
-        acc[1] = fmaf(16.f * __builtin_bit_cast(float, sb.x & 0xffff0000u), d[1], acc[1]);
-        acc[2] = fmaf(16.f * __builtin_bit_cast(float, sb.y << 16), d[2], acc[2]);
-        acc[3] = fmaf(16.f * __builtin_bit_cast(float, sb.y & 0xffff0000u), d[3], acc[3]);
-    }
-    {   // the X_g terms of this wave's 16 groups, one group per column lane
-        const int gg = 16 * wave + n;
-        const uint2 sb = *reinterpret_cast<const uint2 *>(&sc_l[gg][4 * g]);
-        const uint2 bb = *reinterpret_cast<const uint2 *>(&bi_l[gg][4 * g]);
-        const float xg = xsum[gg];
-        const float sv[4] = {__builtin_bit_cast(float, sb.x << 16), __builtin_bit_cast(float, sb.x & 0xffff0000u),
-                             __builtin_bit_cast(float, sb.y << 16), __builtin_bit_cast(float, sb.y & 0xffff0000u)};
-        const float bv[4] = {__builtin_bit_cast(float, bb.x << 16), __builtin_bit_cast(float, bb.x & 0xffff0000u),
-                             __builtin_bit_cast(float, bb.y << 16), __builtin_bit_cast(float, bb.y & 0xffff0000u)};
+        // group 2 st + half of this wave's 16: its scale (lanes g < 2) or bias (the others) for row n
+        const float xg = xs_g[2 * st];
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[i] = fmaf(bv[i] - 16.f * sv[i], xg, acc[i]);
+        for (int T = 0; T < TILES; T++) {
+            const uint32_t word = st < 4 ? q0[T][st & 3] : q1[T][st & 3];
+            const float val = __builtin_bit_cast(float, (word << sh) & 0xffff0000u);
+            const float dsum = (d[T][0] + d[T][1]) + d[T][2];   // sum (1 + nibble/16) x over the group
+            acc[T] = fmaf(val, g < 2 ? 16.f * (dsum - xg) : xg, acc[T]);   // 16 s (D - X_g)  |  b X_g
+        }
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[i] = group_sum<16>(acc[i]);
-    if (n == 0) *reinterpret_cast<mv_f32x4 *>(&red[wave][4 * g]) = mv_f32x4{acc[0], acc[1], acc[2], acc[3]};
+    for (int T = 0; T < TILES; T++) {
+        acc[T] += __shfl_xor(acc[T], 16, 64);
+        acc[T] += __shfl_xor(acc[T], 32, 64);
+        if (g == 0) red[wave][16 * T + n] = acc[T];
+    }
     __syncthreads();
-    if (tid < 16 && row0 + tid < out_dim) {
+    const int row = (t - q.first) * 16 * TILES + tid;
+    if (tid < 16 * TILES && row < q.out_dim) {
         float v = 0.f;
 #pragma unroll
         for (int k = 0; k < WAVES; k++) v += red[k][tid];
-        sp.out[s][row0 + tid] = v;
+        q.out[row] = v;
     }
+}
+
+template <int WAVES, bool SB16>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(5, 8))) void dequant_matvec_mfma_kernel(MatvecSpecs sp, MatvecTiles tl) {
+    dequant_matvec_body<WAVES, SB16, 1>(sp, tl);
 }
 
 // Device pointers; one launch for up to 8 products (the reference batches a layer's
@@ -205,6 +278,7 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
     if (n <= 0 || n > kMvMaxSpecs) return fail(MFA_ERR_INVALID, "dequant matvec: 1 to %d products per call (got %d)", kMvMaxSpecs, n);
     MatvecSpecs sp{};
     int max_out = 0, max_in = 0;
+    bool sb16 = true;   // scale and bias rows can be read 16 bytes at a time in every product
     for (int i = 0; i < n; i++) {
         if (!w[i] || !scales[i] || !biases[i] || !x[i] || !out[i]) return fail(MFA_ERR_INVALID, "dequant matvec: NULL pointer in product %d", i);
         if (out_dim[i] <= 0 || in_dim[i] <= 0) return fail(MFA_ERR_INVALID, "dequant matvec: non-positive shape in product %d", i);
@@ -212,6 +286,9 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
         if (in_dim[i] > 8192) return fail(MFA_ERR_SHAPE, "dequant matvec: in_dim %d > 8192 not supported", in_dim[i]);
         sp.w[i] = w[i]; sp.scales[i] = scales[i]; sp.biases[i] = biases[i]; sp.x[i] = x[i]; sp.out[i] = out[i];
         sp.out_dim[i] = out_dim[i]; sp.in_dim[i] = in_dim[i];
+        if ((uintptr_t)w[i] % 16 != 0 || (uintptr_t)x[i] % 16 != 0)
+            return fail(MFA_ERR_INVALID, "dequant matvec: weights and x of product %d must be 16-byte aligned", i);
+        if ((in_dim[i] / 64) % 8 != 0 || (uintptr_t)scales[i] % 16 != 0 || (uintptr_t)biases[i] % 16 != 0) sb16 = false;
         max_out = out_dim[i] > max_out ? out_dim[i] : max_out;
         max_in = in_dim[i] > max_in ? in_dim[i] : max_in;
     }
@@ -221,10 +298,16 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
     const dim3 grid(tl.first[n]);
     (void)max_out;
     (void)num_cus;
-    if (max_in <= 1024) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<1>), grid, dim3(64), 0, stream, sp, tl, n);
-    else if (max_in <= 2048) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<2>), grid, dim3(128), 0, stream, sp, tl, n);
-    else if (max_in <= 4096) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<4>), grid, dim3(256), 0, stream, sp, tl, n);
-    else hipLaunchKernelGGL((dequant_matvec_mfma_kernel<8>), grid, dim3(512), 0, stream, sp, tl, n);
+#define MV_LAUNCH(W)                                                                                              \
+    do {                                                                                                          \
+        if (sb16) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, true>), grid, dim3(W * 64), 0, stream, sp, tl);   \
+        else hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, false>), grid, dim3(W * 64), 0, stream, sp, tl);       \
+    } while (0)
+    if (max_in <= 1024) MV_LAUNCH(1);
+    else if (max_in <= 2048) MV_LAUNCH(2);
+    else if (max_in <= 4096) MV_LAUNCH(4);
+    else MV_LAUNCH(8);
+#undef MV_LAUNCH
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

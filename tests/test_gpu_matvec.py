@@ -114,6 +114,37 @@ def test_batched_products_of_different_widths(mfa, oracle):
             assert rel_err(o.to_host(), r) <= TOL_F32, sh
 
 
+def test_scale_rows_off_a_16_byte_boundary(mfa, oracle):
+    """Scales and biases that start 2 bytes past a 16-byte boundary take the element-wise loads;
+    the result is the same as for aligned ones."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    rng = np.random.default_rng(9)
+    od, idim = 100, 4096
+    packed, sc, bi = _weights(rng, od, idim, oracle)
+    x = rng.standard_normal(idim).astype(np.float32)
+    ref = oracle.dequant_matvec_4bit(packed, sc, bi, idim, od, x)
+    pad = lambda a: np.concatenate([np.zeros(1, np.uint16), np.ascontiguousarray(a).reshape(-1)])
+    dw, dx = DeviceArray.from_host(packed), DeviceArray.from_host(x)
+    ds, db = DeviceArray.from_host(pad(sc)), DeviceArray.from_host(pad(bi))
+    das, dab = DeviceArray.from_host(np.ascontiguousarray(sc)), DeviceArray.from_host(np.ascontiguousarray(bi))
+    o1, o2 = DeviceArray((od,), np.float32, zero=True), DeviceArray((od,), np.float32, zero=True)
+    with mfa.Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64,
+                        kv_capacity=4)) as c:
+        spec = (ffi.mfa_matvec_spec * 1)(ffi.mfa_matvec_spec(dw.ptr, ds.offset(1), db.offset(1), dx.ptr, o1.ptr, od, idim))
+        assert c.lib.mfa_dequant_matvec_4bit_dev(c.h, 1, C.byref(spec)) == 0, ffi.last_error()
+        spec = (ffi.mfa_matvec_spec * 1)(ffi.mfa_matvec_spec(dw.ptr, das.ptr, dab.ptr, dx.ptr, o2.ptr, od, idim))
+        assert c.lib.mfa_dequant_matvec_4bit_dev(c.h, 1, C.byref(spec)) == 0, ffi.last_error()
+        c.sync()
+        assert rel_err(o1.to_host(), ref) <= TOL_F32
+        assert np.array_equal(o1.to_host(), o2.to_host())
+        # weights and x are read 16 bytes at a time: other alignments are refused, not misread
+        spec = (ffi.mfa_matvec_spec * 1)(ffi.mfa_matvec_spec(dw.offset(1), das.ptr, dab.ptr, dx.ptr, o2.ptr, od - 1, idim))
+        assert c.lib.mfa_dequant_matvec_4bit_dev(c.h, 1, C.byref(spec)) == ffi.ERR_INVALID
+        spec = (ffi.mfa_matvec_spec * 1)(ffi.mfa_matvec_spec(dw.ptr, das.ptr, dab.ptr, dx.offset(1), o2.ptr, od, idim - 64))
+        assert c.lib.mfa_dequant_matvec_4bit_dev(c.h, 1, C.byref(spec)) == ffi.ERR_INVALID
+
+
 def test_matvec_errors(mfa):
     """cpu_matvec.rs:92-97: in_dim must be a multiple of the group size; NULL and shape checks."""
     from moeflux_amd import ffi
