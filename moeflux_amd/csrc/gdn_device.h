@@ -1,6 +1,8 @@
 // Device helpers shared by the Gated-DeltaNet kernels (gdn.hip, gdn_chunk.hip).
 #pragma once
 
+#include <type_traits>
+
 #include "mfa_internal.h"
 
 namespace mfa {
@@ -38,6 +40,24 @@ template <int W> __device__ inline float group_sum(float v) {
             __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
     }
     return v;
+}
+
+// Maximum over the 64 lanes of a wave, in every lane (same data movement as group_sum<64>).
+__device__ inline float wave_max(float v) {
+    auto step = [](float x, auto ctrl) {
+        const int t = __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x),
+                                                  decltype(ctrl)::value, 0xF, 0xF, false);
+        return fmaxf(x, __builtin_bit_cast(float, t));
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});
+    v = step(v, std::integral_constant<int, 0x4E>{});
+    v = step(v, std::integral_constant<int, 0x141>{});
+    v = step(v, std::integral_constant<int, 0x140>{});
+    const int b = __builtin_bit_cast(int, v);
+    return fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)),
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))),
+                 fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)),
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48))));
 }
 
 // Delta-rule update of one state row held by 8 lanes (lane j owns floats

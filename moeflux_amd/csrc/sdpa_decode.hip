@@ -31,6 +31,7 @@
 //     workgroup is written.
 //   sdpa_merge_kernel    log-sum-exp merge of the partials, normalisation and
 //     the sigmoid gate.
+#include "gdn_device.h"
 #include "sdpa_wave.h"
 
 namespace mfa {
@@ -233,70 +234,61 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
 }
 
 // grid (Hq, D/64), 256 threads: 16 lanes x float4 cover 64 outputs of one split's row,
-// 16 such rows per pass.  Each thread's partial rows are requested before the weights
-// are known, so the kernel pays one memory round trip.
+// 16 such rows per pass.  Every wave forms the overall maximum and the denominator by
+// itself (each lane reads the (max, sum) of splits lane, lane + 64, ..., and the maxima of
+// the splits whose rows it combines), so nothing waits for another wave until the 16 row
+// sums meet in LDS, and every request - split statistics, rows, gate - is made before the
+// first value is used: one memory round trip and one barrier.
 static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
-    __shared__ float wsh[kMaxSplits];
-    __shared__ float redf[4];
     __shared__ float4 acc4[16][16];
     // blockIdx.x = token * Hq + head; its row in the kv head's row list is token*hpk + head%hpk
     const int h = blockIdx.x % Hq, tok = blockIdx.x / Hq;
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int dl = tid & 15, sg = tid >> 4;  // 16 float4 lanes x 16 split lanes
     const int d0 = blockIdx.y * 64 + dl * 4;
+    const float *ml = part_ml + pid0 * 32 + n;   // split s: maximum at ml[32 s], sum at ml[32 s + 16]
 
-    // every thread sees (max, sum) of up to 4 splits; nsplit <= kMaxSplits = 4 * 256
-    float ms[4], ls[4];
+    float ms[4], ls[4];   // splits lane + 64 r (the first 256; beyond that, see the loops below)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int s = tid + 256 * r;
-        ms[r] = (s < nsplit) ? part_ml[(pid0 + s) * 32 + n] : neg_inf();
-        ls[r] = (s < nsplit) ? part_ml[(pid0 + s) * 32 + 16 + n] : 0.f;
+        const int s = lane + 64 * r;
+        ms[r] = (s < nsplit) ? ml[(size_t)s * 32] : neg_inf();
+        ls[r] = (s < nsplit) ? ml[(size_t)s * 32 + 16] : 0.f;
     }
+    float mo[kMergeRows];   // maxima of the splits whose rows this thread combines
     float4 rows[kMergeRows];
 #pragma unroll
     for (int r = 0; r < kMergeRows; r++) {
         const int s = sg + 16 * r;
+        mo[r] = (s < nsplit) ? ml[(size_t)s * 32] : neg_inf();
         rows[r] = (s < nsplit) ? *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0)
                                : float4{0.f, 0.f, 0.f, 0.f};
     }
     const float gt_in = (gate && tid < 64) ? gate[(size_t)blockIdx.x * D + blockIdx.y * 64 + tid] : 0.f;
 
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
-#pragma unroll
-    for (int x = 1; x < 64; x <<= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
-    if (lane == 0) redf[wave] = m;
-    __syncthreads();
-    const float M = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
-    __syncthreads();
+    for (int s = lane + 256; s < nsplit; s += 64) m = fmaxf(m, ml[(size_t)s * 32]);
+    const float M = wave_max(m);
+    auto weight = [&](float ms_) { return (ms_ == neg_inf()) ? 0.f : fast_exp2(ms_ - M); };
     float den = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int s = tid + 256 * r;
-        const float ws = (ms[r] == neg_inf()) ? 0.f : fast_exp2(ms[r] - M);
-        if (s < nsplit) wsh[s] = ws;
-        den += ws * ls[r];
-    }
-#pragma unroll
-    for (int x = 1; x < 64; x <<= 1) den += __shfl_xor(den, x, 64);
-    if (lane == 0) redf[wave] = den;
-    __syncthreads();
-    den = redf[0] + redf[1] + redf[2] + redf[3];
+    for (int r = 0; r < 4; r++) den += weight(ms[r]) * ls[r];
+    for (int s = lane + 256; s < nsplit; s += 64) den += weight(ml[(size_t)s * 32]) * ml[(size_t)s * 32 + 16];
+    den = group_sum<64>(den);
 
     float4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < kMergeRows; r++) {
-        const int s = sg + 16 * r;
-        const float w = (s < nsplit) ? wsh[s] : 0.f;
+        const float w = weight(mo[r]);
         acc.x += w * rows[r].x; acc.y += w * rows[r].y; acc.z += w * rows[r].z; acc.w += w * rows[r].w;
     }
     for (int s = sg + 16 * kMergeRows; s < nsplit; s += 16) {
-        const float w = wsh[s];
+        const float w = weight(ml[(size_t)s * 32]);
         const float4 v = *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0);
         acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
     }
