@@ -56,9 +56,10 @@ __device__ inline wy_f32x4 load_v4(const float *p) { return *reinterpret_cast<co
 //   eL [64] (e^{L_t}; eL[63] = e^{L_C} because padded tokens do not decay).
 // Tokens past the end of the chunk are padded with beta = 0, log g = 0, k = q = v = 0.
 //
-// grid (Hv, blocks), 256 threads.
+// grid (Hv, blocks), one wave per 16 columns of K (DK/16 waves: two per SIMD at DK = 128, so that one
+// has matrix work while the other waits for LDS or stores a tile).
 template <int DK>
-__global__ __launch_bounds__(256) void gdn_wy_kernel(
+__global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ kn,
     const float *__restrict__ vv, const float *__restrict__ lg, const float *__restrict__ bg,
     float *__restrict__ Wt, float *__restrict__ Qt, float *__restrict__ Ut, float *__restrict__ Mt,
@@ -67,7 +68,9 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     constexpr int NK = DK / 16;
     constexpr int LDK = DK + 4;  // row strides chosen so that 16-byte row reads by 8 lanes hit all banks
     constexpr int LDC = kC + 4;
-    constexpr int NCT = DK / 64;  // 16-wide column tiles of W (and of U) per wave
+    constexpr int NW = NK;        // waves
+    constexpr int NTHR = 64 * NW;
+    constexpr int NCT = 1;        // 16-wide column tiles of W (and of U) per wave
     __shared__ __align__(16) float sK[kC][LDK];
     __shared__ __align__(16) float sQ[kC][LDK];  // q^, later v
     __shared__ __align__(16) float sA[kC][LDC];
@@ -84,33 +87,46 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     const size_t slot = (size_t)blk * Hv + vh;
 
     // ---- phase 0: k^, q^ of the block, cumulative log decay, beta ---------------------
+    // Everything the block reads is requested here, in the order of use (loads return in the
+    // order of their requests): the gates, k^ and q^, and v, which waits in registers for phase 2.
+    float lg_in = 0.f, bg_in = 0.f;
+    if (wave == 0 && lane < nt) {
+        lg_in = lg[(size_t)(t0 + lane) * Hv + vh];
+        bg_in = bg[(size_t)(t0 + lane) * Hv + vh];
+    }
+    constexpr int NLV = kC * (DV / 4) / NTHR;
+    float4 va[NLV];
     {
-        // all of a thread's requests go out before the first of them is stored
-        constexpr int NL = kC * (DK / 4) / 256;
+        constexpr int NL = kC * (DK / 4) / NTHR;
         float4 a[NL], b[NL];
 #pragma unroll
         for (int u = 0; u < NL; u++) {
-            const int i = tid + u * 256, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
+            const int i = tid + u * NTHR, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
             const size_t src = ((size_t)(t0 + (tt < nt ? tt : nt - 1)) * Hk + kh) * DK + x;
             a[u] = load_f4(kn + src);
             b[u] = load_f4(qn + src);
         }
 #pragma unroll
+        for (int u = 0; u < NLV; u++) {
+            const int i = tid + u * NTHR, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
+            va[u] = load_f4(vv + ((size_t)(t0 + (tt < nt ? tt : nt - 1)) * Hv + vh) * DV + x);
+        }
+#pragma unroll
         for (int u = 0; u < NL; u++) {
-            const int i = tid + u * 256, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
+            const int i = tid + u * NTHR, tt = i / (DK / 4), x = (i % (DK / 4)) * 4;
             const float keep = tt < nt ? 1.f : 0.f;  // padded tokens are zero rows
             *(float4 *)&sK[tt][x] = float4{a[u].x * keep, a[u].y * keep, a[u].z * keep, a[u].w * keep};
             *(float4 *)&sQ[tt][x] = float4{b[u].x * keep, b[u].y * keep, b[u].z * keep, b[u].w * keep};
         }
     }
     if (wave == 0) {
-        float l = lane < nt ? lg[(size_t)(t0 + lane) * Hv + vh] : 0.f;
+        float l = lg_in;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
             const float u = __shfl_up(l, d, 64);
             if (lane >= d) l += u;
         }
-        const float b = lane < nt ? bg[(size_t)(t0 + lane) * Hv + vh] : 0.f;
+        const float b = bg_in;
         sL[lane] = l;
         sB[lane] = b;
         sCw[lane] = b * expf(l);
@@ -120,10 +136,12 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     __syncthreads();
 
     // ---- phase 1: the lower tiles of K K^T (-> A) and of Q K^T (-> M) -----------------
-    // 10 tiles (I, J <= I) each; 20 jobs of DK/4 instructions over 4 waves.
+    // 10 tiles (I, J <= I) each; 20 jobs of DK/4 instructions dealt round the waves.
 #pragma unroll
-    for (int r = 0; r < 5; r++) {
-        const int job = wave * 5 + r, kind = job / 10, idx = job % 10;
+    for (int r = 0; r < (20 + NW - 1) / NW; r++) {
+        const int job = wave + NW * r;
+        if (job >= 20) break;   // uniform over the wave
+        const int kind = job / 10, idx = job % 10;
         const int I = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
         const int J = idx - I * (I + 1) / 2;
         const float(*X)[LDK] = kind ? sQ : sK;
@@ -143,7 +161,7 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
                 Mt[((slot * 4 + I) * 4 + J) * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = (col <= row) ? d * acc[i] : 0.f;
         }
     }
-    for (int i = tid; i < 4 * NK * 64; i += 256) {  // q^ tiles, before v takes its place
+    for (int i = tid; i < 4 * NK * 64; i += NTHR) {  // q^ tiles, before v takes its place
         const int tile = i >> 6, l = i & 63, w = tile / NK, c = tile % NK;
         *(float4 *)(Qt + (slot * 4 * NK + tile) * 256 + l * 4) = lds_f4(&sQ[16 * w + (l & 15)][16 * c + 4 * (l >> 4)]);
     }
@@ -154,29 +172,22 @@ __global__ __launch_bounds__(256) void gdn_wy_kernel(
     //      per wave, a column per lane), the blocks below them level by level from
     //      T_IJ = -T_II sum_{J <= K < I} A_IK T_KJ on the matrix cores -----------------------
     {
-        constexpr int NL = kC * (DV / 4) / 256;
-        float4 a[NL];
 #pragma unroll
-        for (int u = 0; u < NL; u++) {
-            const int i = tid + u * 256, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
-            a[u] = load_f4(vv + ((size_t)(t0 + (tt < nt ? tt : nt - 1)) * Hv + vh) * DV + x);
-        }
-#pragma unroll
-        for (int u = 0; u < NK * 4 * 64 / 256; u++) {
-            const int i = tid + u * 256, tile = i >> 6, l = i & 63, c = tile >> 2, tau = tile & 3;
+        for (int u = 0; u < NK * 4 * 64 / NTHR; u++) {
+            const int i = tid + u * NTHR, tile = i >> 6, l = i & 63, c = tile >> 2, tau = tile & 3;
             const int kk = 16 * c + (l & 15), j4 = 16 * tau + 4 * (l >> 4);
             const float4 e = lds_f4(&sKd[j4]);
             const float4 o = {e.x * sK[j4 + 0][kk], e.y * sK[j4 + 1][kk], e.z * sK[j4 + 2][kk], e.w * sK[j4 + 3][kk]};
             *(float4 *)(Kt + (slot * NK * 4 + tile) * 256 + l * 4) = o;
         }
 #pragma unroll
-        for (int u = 0; u < NL; u++) {
-            const int i = tid + u * 256, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
+        for (int u = 0; u < NLV; u++) {
+            const int i = tid + u * NTHR, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
             const float keep = tt < nt ? 1.f : 0.f;
-            *(float4 *)&sQ[tt][x] = float4{a[u].x * keep, a[u].y * keep, a[u].z * keep, a[u].w * keep};
+            *(float4 *)&sQ[tt][x] = float4{va[u].x * keep, va[u].y * keep, va[u].z * keep, va[u].w * keep};
         }
     }
-    {
+    if (wave < 4) {
         // block `wave`; the four lane groups compute the same 16 columns, group 0 stores
         const int r0 = 16 * wave;
         float t[16];
@@ -412,7 +423,7 @@ int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const fl
     float *Mt = Ut + slots * kC * dv;
     float *eLc = Mt + slots * kC * kC;
     if (dk == 128) {
-        hipLaunchKernelGGL((gdn_wy_kernel<128>), dim3(Hv, (unsigned)nblk), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
+        hipLaunchKernelGGL((gdn_wy_kernel<128>), dim3(Hv, (unsigned)nblk), dim3(512), 0, s, Hk, Hv, T, qn, kn, vv,
                            lg, bg, Wt, Qt, Ut, Mt, Kt, eLc);
         hipLaunchKernelGGL((gdn_wy_recur_kernel<128>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, Wt, Qt, Ut,
                            Mt, Kt, eLc, ssm, o_raw);
