@@ -344,6 +344,10 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
             fetch_wq(blk + 1, c);
 #pragma unroll
             for (int u = 0; u < LATE_PER_C; u++) fetch_late(nxt, blk + 1, c * LATE_PER_C + u);
+            // keep this column tile's requests between its matrix instructions (left to itself the
+            // scheduler gathers all requests at the end of the product, where nothing hides their issue)
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 2 + LATE_PER_C, 0);
         }
         // ---- D = U - W S0^T: lane (n, g) holds tokens 16w+4g+i of state row row0+n ----
         wy_f32x4 d;
