@@ -342,11 +342,17 @@ static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, in
     const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
     int64_t target = forced > 0 ? forced : (num_cus / ((int64_t)Hkv * p.nhg));
     if (target < 1) target = 1;
+    // Up to head_dim 128 two 8-wave workgroups fit a CU (<= 128 registers): give every CU two
+    // where each still gets a whole pass of 8 blocks (f32, d=128, 32K: 25.6 -> 23.5 us).
+    if (forced <= 0 && D <= 128 && nblk >= 8 * 2 * target) target *= 2;
     if (target > kMaxSplits) target = kMaxSplits;
     p.bps = (nblk + target - 1) / target;
     if (p.bps < 1) p.bps = 1;
     p.waves = (p.bps >= 8 && D >= 128) ? 8 : 4;
-    if (forced <= 0 && p.bps < p.waves) p.bps = p.waves;  // at least one block per wave
+    // Whole super-blocks only (one block per wave and pass): a pass with idle waves costs as
+    // much as a full one, and fewer workgroups of full passes measured 12-18 % faster than
+    // one workgroup per CU with a ragged last pass (kv_len 20K-48K at 2 kv heads).
+    if (forced <= 0) p.bps = (p.bps + p.waves - 1) / p.waves * p.waves;
     p.splits = (int)((nblk + p.bps - 1) / p.bps);
     if (p.splits < 1) p.splits = 1;
     return p;
