@@ -351,6 +351,26 @@ def bench_matvec(steps, warmup, seed):
         alg = nw // 2 + (nw // 64) * 4 + idim * 4 + sum(shapes) * 4
         res[name] = {"shapes": [[od, idim] for od in shapes], "us_per_launch": ev_ms * 1e3, "algorithmic_bytes": alg,
                      "gbps": alg / (ev_ms * 1e-3) / 1e9, "pct_peak": 100.0 * alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        # the same products over weights re-ordered at load time (mfa_matvec_tile_weights_dev)
+        tsets = []
+        for specs in sets:
+            tspecs = (ffi.mfa_matvec_spec * len(shapes))()
+            for i, od in enumerate(shapes):
+                tw = DeviceArray((int(lib.mfa_matvec_tiled_words(od, idim)),), np.uint32)
+                keep.append(tw)
+                if lib.mfa_matvec_tile_weights_dev(ctx.h, od, idim, specs[i].w_packed, tw.ptr) != 0:
+                    raise RuntimeError(ffi.last_error())
+                sp = specs[i]
+                tspecs[i] = ffi.mfa_matvec_spec(tw.ptr, sp.scales, sp.biases, sp.x, sp.out, od, idim)
+            tsets.append(tspecs)
+
+        def tstep(i, tsets=tsets, n=len(shapes)):
+            if lib.mfa_dequant_matvec_4bit_tiled_dev(ctx.h, n, C.byref(tsets[i % len(tsets)])) != 0:
+                raise RuntimeError(ffi.last_error())
+
+        wall_ms, ev_ms = _timed(ctx, lib, tstep, steps, warmup)
+        res[name]["tiled_weights_us_per_launch"] = ev_ms * 1e3
+        res[name]["tiled_weights_pct_peak"] = 100.0 * alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS
     ctx.close()
     for a in keep:
         a.free()

@@ -836,7 +836,7 @@ int mfa_mla_sdpa_folded(int32_t num_heads, int32_t kv_lora_rank, int32_t qk_rope
 
 /* ---- projections ------------------------------------------------------------------- */
 
-int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs) {
+static int matvec_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs, bool tiled) {
     Ctx *c = as_ctx(ctx);
     if (!c || !specs) return fail(MFA_ERR_INVALID, "NULL argument");
     if (n <= 0 || n > 8) return fail(MFA_ERR_INVALID, "1 to 8 products per call (got %d)", n);
@@ -849,7 +849,26 @@ int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *
         w[i] = specs[i].w_packed; sc[i] = specs[i].scales; bi[i] = specs[i].biases;
         x[i] = specs[i].x; out[i] = specs[i].out; od[i] = specs[i].out_dim; id[i] = specs[i].in_dim;
     }
-    return launch_dequant_matvec_4bit(c->stream, n, w, sc, bi, x, out, od, id, c->num_cus);
+    return launch_dequant_matvec_4bit(c->stream, n, w, sc, bi, x, out, od, id, c->num_cus, tiled);
+}
+
+int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs) {
+    return matvec_dev(ctx, n, specs, false);
+}
+
+int mfa_dequant_matvec_4bit_tiled_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs) {
+    return matvec_dev(ctx, n, specs, true);
+}
+
+int64_t mfa_matvec_tiled_words(int32_t out_dim, int32_t in_dim) {
+    if (out_dim <= 0 || in_dim <= 0 || in_dim % 64 != 0) return fail(MFA_ERR_INVALID, "out_dim %d, in_dim %d (a multiple of 64)", out_dim, in_dim);
+    return (int64_t)matvec_tiled_words(out_dim, in_dim);
+}
+
+int mfa_matvec_tile_weights_dev(mfa_ctx *ctx, int32_t out_dim, int32_t in_dim, const uint32_t *w_packed, uint32_t *w_tiled) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    return launch_matvec_tile_weights(c->stream, out_dim, in_dim, w_packed, w_tiled);
 }
 
 int mfa_dequant_matvec_4bit(int32_t out_dim, int32_t in_dim, int32_t group_size, const uint32_t *w_packed,

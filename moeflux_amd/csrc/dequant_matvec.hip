@@ -104,7 +104,7 @@ __device__ inline Product mv_product_of(const MatvecSpecs &sp, const MatvecTiles
 // Loads come back in the order they were asked for, so the order of the requests is the order
 // of use: x (staged in LDS while everything else is on its way), the row's scales and biases
 // (16 bytes per lane straight into registers), then the 8 x 16 bytes of weights per lane.
-template <int WAVES, bool SB16, int TILES>
+template <int WAVES, bool SB16, int TILES, bool TILED>
 __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const MatvecTiles &tl) {
     constexpr int KP = WAVES * 1024;   // inputs covered by the workgroup (in_dim padded)
     constexpr int G = KP / 64;         // scale groups
@@ -138,8 +138,15 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
             const int c = 4 * (wave * STEPS + st) + g;
 #pragma unroll
             for (int T = 0; T < TILES; T++) {
-                const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
-                w[T][st] = *reinterpret_cast<const mv_u32x4 *>(q.w + (size_t)row * words + (c < nchunk ? c : 0) * 4);  // past the row: any chunk, x is 0 there
+                if constexpr (TILED) {
+                    // [tile][run of 1024 inputs][step][lane]: a wave's request is 1 KiB in one piece
+                    const int nruns = (in_dim + 1023) >> 10, tile = (t - q.first) * TILES + T;
+                    const size_t at = (((size_t)tile * nruns + (wave < nruns ? wave : 0)) * STEPS + st) * 64 + lane;
+                    w[T][st] = *reinterpret_cast<const mv_u32x4 *>(q.w + at * 4);
+                } else {
+                    const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
+                    w[T][st] = *reinterpret_cast<const mv_u32x4 *>(q.w + (size_t)row * words + (c < nchunk ? c : 0) * 4);  // past the row: any chunk, x is 0 there
+                }
             }
         }
     };
@@ -265,16 +272,48 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
     }
 }
 
-template <int WAVES, bool SB16>
+template <int WAVES, bool SB16, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(5, 8))) void dequant_matvec_mfma_kernel(MatvecSpecs sp, MatvecTiles tl) {
-    dequant_matvec_body<WAVES, SB16, 1>(sp, tl);
+    dequant_matvec_body<WAVES, SB16, 1, TILED>(sp, tl);
+}
+
+// Weights re-ordered for the kernel above, once, when a model is loaded: for every 16-row tile
+// and every run of 1024 inputs the 8 x 64 x 16 bytes its wave requests, in request order
+// (step, then lane: row lane % 16, 32-input chunk 4 (8 run + step) + lane / 16).  Rows past
+// out_dim repeat the last row, chunks past in_dim are zero.  grid (runs, tiles), 512 threads.
+__global__ __launch_bounds__(512) void matvec_tile_weights_kernel(const uint32_t *__restrict__ w, uint32_t *__restrict__ tiled,
+                                                                  int out_dim, int in_dim) {
+    const int run = blockIdx.x, tile = blockIdx.y, nruns = gridDim.x;
+    const int st = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = min(16 * tile + (lane & 15), out_dim - 1);
+    const int c = 4 * (8 * run + st) + (lane >> 4);
+    mv_u32x4 v = {0u, 0u, 0u, 0u};
+    if (c < (in_dim >> 5)) v = *reinterpret_cast<const mv_u32x4 *>(w + (size_t)row * (in_dim >> 3) + 4 * c);
+    *reinterpret_cast<mv_u32x4 *>(tiled + ((((size_t)tile * nruns + run) * 8 + st) * 64 + lane) * 4) = v;
+}
+
+size_t matvec_tiled_words(int out_dim, int in_dim) {
+    return (size_t)((out_dim + 15) / 16) * ((in_dim + 1023) / 1024) * 8 * 64 * 4;
+}
+
+int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, uint32_t *tiled) {
+    if (!w || !tiled) return fail(MFA_ERR_INVALID, "matvec tiling: NULL argument");
+    if (out_dim <= 0 || in_dim <= 0 || in_dim % 64 != 0)
+        return fail(MFA_ERR_INVALID, "matvec tiling: out_dim %d, in_dim %d (a multiple of 64)", out_dim, in_dim);
+    if ((uintptr_t)w % 16 != 0 || (uintptr_t)tiled % 16 != 0)
+        return fail(MFA_ERR_INVALID, "matvec tiling: weights must be 16-byte aligned");
+    if ((out_dim + 15) / 16 > 65535) return fail(MFA_ERR_SHAPE, "matvec tiling: out_dim %d too large", out_dim);
+    hipLaunchKernelGGL(matvec_tile_weights_kernel, dim3((in_dim + 1023) / 1024, (out_dim + 15) / 16), dim3(512), 0, stream,
+                       w, tiled, out_dim, in_dim);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
 }
 
 // Device pointers; one launch for up to 8 products (the reference batches a layer's
 // projections into one command buffer, full_attn_forward.rs:193-227).
 int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const *w, const uint16_t *const *scales,
                                const uint16_t *const *biases, const float *const *x, float *const *out,
-                               const int *out_dim, const int *in_dim, int num_cus) {
+                               const int *out_dim, const int *in_dim, int num_cus, bool tiled) {
     if (n <= 0 || n > kMvMaxSpecs) return fail(MFA_ERR_INVALID, "dequant matvec: 1 to %d products per call (got %d)", kMvMaxSpecs, n);
     MatvecSpecs sp{};
     int max_out = 0, max_in = 0;
@@ -300,8 +339,10 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
     (void)num_cus;
 #define MV_LAUNCH(W)                                                                                              \
     do {                                                                                                          \
-        if (sb16) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, true>), grid, dim3(W * 64), 0, stream, sp, tl);   \
-        else hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, false>), grid, dim3(W * 64), 0, stream, sp, tl);       \
+        if (sb16 && tiled) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, true, true>), grid, dim3(W * 64), 0, stream, sp, tl);   \
+        else if (sb16) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, true, false>), grid, dim3(W * 64), 0, stream, sp, tl);      \
+        else if (tiled) hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, false, true>), grid, dim3(W * 64), 0, stream, sp, tl);     \
+        else hipLaunchKernelGGL((dequant_matvec_mfma_kernel<W, false, false>), grid, dim3(W * 64), 0, stream, sp, tl);               \
     } while (0)
     if (max_in <= 1024) MV_LAUNCH(1);
     else if (max_in <= 2048) MV_LAUNCH(2);

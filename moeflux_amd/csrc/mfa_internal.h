@@ -207,7 +207,10 @@ int launch_mla_sdpa_folded(hipStream_t stream, int H, int R, int P, int L, float
 // dequant_matvec.hip: up to 8 four-bit dequantising matrix-vector products in one launch.
 int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const *w, const uint16_t *const *scales,
                                const uint16_t *const *biases, const float *const *x, float *const *out,
-                               const int *out_dim, const int *in_dim, int num_cus = 256);
+                               const int *out_dim, const int *in_dim, int num_cus = 256, bool tiled = false);
+// The weight order the tiled form of the kernel reads (words of the re-ordered copy, and the copy itself).
+size_t matvec_tiled_words(int out_dim, int in_dim);
+int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, uint32_t *tiled);
 // attn_prologue.hip: q/gate split, per-head norms, rotation, cache append of one token.
 int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
                          int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,

@@ -145,6 +145,61 @@ def test_scale_rows_off_a_16_byte_boundary(mfa, oracle):
         assert c.lib.mfa_dequant_matvec_4bit_dev(c.h, 1, C.byref(spec)) == ffi.ERR_INVALID
 
 
+def test_tiled_weights_give_the_same_products(mfa, oracle):
+    """Weights re-ordered on the device (mfa_matvec_tile_weights_dev) and multiplied with
+    mfa_dequant_matvec_4bit_tiled_dev: the same results, bit for bit, as the file order gives, for
+    ragged row counts, input widths that do not fill a run of 1024, and products of different
+    widths in one launch; the re-ordered copy itself is checked against the layout's definition."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    rng = np.random.default_rng(10)
+    shapes = [(100, 4096), (33, 64), (512, 2048), (1, 1024), (17, 4160), (250, 3072), (16, 8192), (1000, 4096)]
+    keep, refs, outs, touts = [], [], [], []
+    specs = (ffi.mfa_matvec_spec * len(shapes))()
+    tspecs = (ffi.mfa_matvec_spec * len(shapes))()
+    with mfa.Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=8, num_kv_heads=2, head_dim=64,
+                        kv_capacity=4)) as c:
+        lib = c.lib
+        for i, (od, idim) in enumerate(shapes):
+            packed, sc, bi = _weights(rng, od, idim, oracle)
+            x = rng.standard_normal(idim).astype(np.float32)
+            refs.append(oracle.dequant_matvec_4bit(packed, sc, bi, idim, od, x))
+            dw, ds, db, dx = (DeviceArray.from_host(a) for a in (packed, sc, bi, x))
+            words = int(lib.mfa_matvec_tiled_words(od, idim))
+            tiles, runs = (od + 15) // 16, (idim + 1023) // 1024
+            assert words == tiles * runs * 8 * 64 * 4
+            dt = DeviceArray((words,), np.uint32)
+            assert lib.mfa_matvec_tile_weights_dev(c.h, od, idim, dw.ptr, dt.ptr) == 0, ffi.last_error()
+            do, dto = DeviceArray((od,), np.float32, zero=True), DeviceArray((od,), np.float32, zero=True)
+            keep += [dw, ds, db, dx, dt]
+            outs.append(do)
+            touts.append(dto)
+            specs[i] = ffi.mfa_matvec_spec(dw.ptr, ds.ptr, db.ptr, dx.ptr, do.ptr, od, idim)
+            tspecs[i] = ffi.mfa_matvec_spec(dt.ptr, ds.ptr, db.ptr, dx.ptr, dto.ptr, od, idim)
+            if i in (0, 4):   # the layout: [tile][run][step][lane] x 4 words
+                c.sync()
+                t = dt.to_host().reshape(tiles, runs, 8, 64, 4)
+                shape4 = (tiles, runs, 8, 64)
+                rows = np.broadcast_to(np.minimum(16 * np.arange(tiles)[:, None, None, None] + np.arange(64)[None, None, None, :] % 16, od - 1), shape4)
+                chunk = np.broadcast_to(4 * (8 * np.arange(runs)[None, :, None, None] + np.arange(8)[None, None, :, None]) + np.arange(64)[None, None, None, :] // 16, shape4)
+                src = np.zeros((od, runs * 32, 4), np.uint32)
+                src[:, :idim // 32] = packed.reshape(od, idim // 32, 4)
+                assert np.array_equal(t, src[rows, chunk])
+        assert lib.mfa_dequant_matvec_4bit_dev(c.h, len(shapes), C.byref(specs)) == 0, ffi.last_error()
+        assert lib.mfa_dequant_matvec_4bit_tiled_dev(c.h, len(shapes), C.byref(tspecs)) == 0, ffi.last_error()
+        c.sync()
+        for o, to, r, sh in zip(outs, touts, refs, shapes):
+            assert rel_err(to.to_host(), r) <= TOL_F32, sh
+            assert np.array_equal(o.to_host(), to.to_host()), sh
+        # aligned group counts only (the 16-byte scale loads), one product
+        one = (ffi.mfa_matvec_spec * 1)(tspecs[7])
+        assert lib.mfa_dequant_matvec_4bit_tiled_dev(c.h, 1, C.byref(one)) == 0, ffi.last_error()
+        c.sync()
+        assert np.array_equal(touts[7].to_host(), outs[7].to_host())
+        assert lib.mfa_matvec_tiled_words(16, 32) < 0
+        assert lib.mfa_matvec_tile_weights_dev(c.h, 16, 64, None, keep[4].ptr) == ffi.ERR_INVALID
+
+
 def test_matvec_errors(mfa):
     """cpu_matvec.rs:92-97: in_dim must be a multiple of the group size; NULL and shape checks."""
     from moeflux_amd import ffi

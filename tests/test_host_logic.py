@@ -68,7 +68,14 @@ def test_split_partitioning():
     for forced in (1, 2, 7, 64):
         got = ns(ffi.KV_BF16, 32, 2, 256, 8192, 256, forced)
         assert 1 <= got <= forced
-    # more than 16 query heads per kv head: head groups share the CUs
-    assert ns(ffi.KV_BF16, 64, 2, 128, 32768, 256, 0) == 64
+    # more than 16 query heads per kv head: head groups share the CUs; up to head_dim 128 two
+    # workgroups fit a CU, so 2 * 256 / 4 splits where each still gets a whole pass of 8 blocks
+    assert ns(ffi.KV_BF16, 64, 2, 128, 32768, 256, 0) == 128
+    assert ns(ffi.KV_F32, 32, 4, 128, 32768, 256, 0) == 128       # 2048 blocks of 16, 16 per split
+    assert ns(ffi.KV_F32, 32, 4, 128, 8192, 256, 0) == 64         # 512 blocks: one pass of 8 each, not doubled
+    # whole passes only: 12 layers x 2 kv heads of 256 blocks -> 256 / 24 = 10 splits of 26 blocks
+    # would leave a ragged fourth pass; 8 splits of 32
+    assert ns(ffi.KV_BF16, 32 * 12, 2 * 12, 256, 8192, 256, 0) == 8
+    assert ns(ffi.KV_BF16, 32, 2, 256, 49152, 256, 0) == 96       # 1536 blocks: 16 per split, not 12
     assert ns(ffi.KV_BF16, 30, 4, 128, 64, 256, 0) == -1          # 30 % 4 != 0
     assert ns(ffi.KV_BF16, 32, 2, 256, 0, 256, 0) == -1
