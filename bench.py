@@ -1,11 +1,12 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X attention path.
 
-Headline (the one JSON line the driver reads): BASELINE.json's metric, attention
+Headline (the one JSON line the driver reads): attention
 microseconds per layer per token with the achieved HBM rate, on the
 long-context configuration the metric is quoted on — gated GQA decode,
 32 Q / 2 KV heads, head_dim 256, 32768 cached positions, bf16 K/V, batch 1
-(configs[2]; configs[0] and [1] are reported under "extra").  A "step" is one
+(the other workloads - 4K f32 decode, the DeltaNet step, the 512-token chunk, the 48-layer
+sweep, the projections and the latent-cache attention - are reported under "extra").  A "step" is one
 layer's decode attention for one token: mfa_sdpa_decode_dev over a KV cache that
 already resides in HBM.  Steps rotate over `--layers` independent caches whose
 total exceeds the 256 MB last-level cache, so every step streams from HBM.
@@ -149,7 +150,7 @@ def bench_gdn(name, Hk, Hv, dk, dv, layers, steps, warmup, seed):
 
 
 def bench_prefill(steps, warmup, seed, T=512):
-    """BASELINE configs[3]: a 512-token prompt chunk from an empty cache / zero state —
+    """A 512-token prompt chunk from an empty cache / zero state —
     causal GQA attention (32 Q / 4 KV heads, d=128, bf16 cache) and the Gated-DeltaNet
     chunk (configs[1] shape).  Every timed call uses a fresh layer, so kv_len0 = 0."""
     from moeflux_amd import Config, Ctx, ffi
@@ -210,7 +211,7 @@ def bench_prefill(steps, warmup, seed, T=512):
 
 
 def bench_sweep(steps, warmup, seed):
-    """BASELINE configs[4]: the attention launches of one token over a 48-layer hybrid stack,
+    """The attention launches of one token over a 48-layer hybrid stack,
     36 Gated-DeltaNet layers (configs[1] shape) and 12 gated full-attention layers
     (32 Q / 2 KV heads, d=256, kv_len 8192, bf16), distinct buffers per layer, in layer order
     on one stream (mfa_token_sweep_dev)."""

@@ -34,7 +34,7 @@ def test_gdn_step_matches_oracle(mfa, Hk, Hv, dk, dv):
 
 
 def test_config2_from_zero_state_and_prefill(mfa):
-    """BASELINE config 2 shape with A_log = dt_bias = 0 and unit norm weight; the
+    """The 16 / 32-head, dk = dv = 128 step shape with A_log = dt_bias = 0 and unit norm weight; the
     chunk call equals the token loop."""
     case = GdnCase(0xC0FFEE + 2, 16, 32, 128, 128, T=9, zero_state=True, plain=True)
     ref_out, ref_conv, ref_ssm = case.oracle()
@@ -141,7 +141,7 @@ def test_chunk_blocked_form_dk64(mfa, T):
 
 
 def test_config4_gdn_chunk_of_512_from_zero_state(mfa):
-    """BASELINE config 4, DeltaNet half: 512 tokens of the config-2 shape from a zero state,
+    """The DeltaNet half of the 512-token prompt chunk: 512 tokens of the 16 / 32-head step shape from a zero state,
     against 512 sequential oracle steps; outputs and the final state."""
     case = GdnCase(0xC0FFEE + 4, 16, 32, 128, 128, T=512, zero_state=True)
     ref_out, ref_conv, ref_ssm = case.oracle()

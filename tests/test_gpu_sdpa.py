@@ -39,7 +39,7 @@ def test_sdpa_reference_test_inputs(mfa, oracle, kv_len):
 
 
 def test_config1_full_size(mfa, oracle):
-    """BASELINE config 1: 32 Q / 4 KV heads, d=128, L=4096, fp32."""
+    """The 4K f32 decode shape: 32 Q / 4 KV heads, d=128, L=4096, fp32."""
     Hq, Hkv, d, L = 32, 4, 128, 4096
     q, g, k, v = sdpa_random_inputs(0xC0FFEE + 1, Hq, Hkv, d, L)
     ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
@@ -105,7 +105,7 @@ def test_ctx_append_decode_and_split_invariance(mfa, oracle, bf16):
 
 
 def test_config3_full_size_bf16(mfa, oracle):
-    """BASELINE config 3: 32 Q / 2 KV heads, d=256, L=32768, bf16 K/V, via bulk import."""
+    """The 32K bf16 decode shape (the headline workload): 32 Q / 2 KV heads, d=256, L=32768, bf16 K/V, via bulk import."""
     Hq, Hkv, d, L = 32, 2, 256, 32768
     q, g, k, v = sdpa_random_inputs(0xC0FFEE + 3, Hq, Hkv, d, L, bf16=True)
     ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)

@@ -83,7 +83,7 @@ def test_prefill_attn_shapes(mfa, oracle, Hq, Hkv, d, T, L0, bf16):
 
 
 def test_prefill_attn_bf16_chunk_of_512(mfa, oracle):
-    """BASELINE config 4, attention half: 512 tokens, 32 Q / 4 KV heads, d=128, bf16 values,
+    """The attention half of the 512-token prompt chunk: 512 tokens, 32 Q / 4 KV heads, d=128, bf16 values,
     from an empty cache."""
     Hq, Hkv, d, T = 32, 4, 128, 512
     rng = np.random.default_rng(0xC0FFEE + 4)

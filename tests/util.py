@@ -66,7 +66,7 @@ class GdnCase:
         self.C = C = 2 * Hk * dk + Hv * dv
         self.eps = 1e-6
         self.conv_w = cref.f32_to_bf16(rng.standard_normal(C * K) * 0.5)
-        if plain:  # BASELINE config 2: A_log = 0, dt_bias = 0, norm weight = 1
+        if plain:  # the plain step shape: A_log = 0, dt_bias = 0, norm weight = 1
             self.a_log = np.zeros(Hv, np.float32)
             self.dt_bias = cref.f32_to_bf16(np.zeros(Hv))
             self.norm_w = cref.f32_to_bf16(np.ones(dv))
