@@ -38,6 +38,26 @@ def test_sdpa_reference_test_inputs(mfa, oracle, kv_len):
     assert rel_err(out, ref) <= TOL_F32
 
 
+def test_sdpa_random_shapes_default_split_planning(mfa, oracle):
+    """Seeded random shapes and lengths through the default split planning (whole passes per
+    workgroup, two workgroups per CU up to head_dim 128): lengths around pass and block edges,
+    every head_dim, f32 and bf16 caches."""
+    rng = np.random.default_rng(2024)
+    edges = [255, 256, 257, 2047, 2048, 2049, 4095, 4097, 6143, 6145, 8191, 8193, 12289, 16383, 16385, 20481]
+    for case in range(28):
+        d = int(rng.choice([64, 128, 256]))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        hpk = int(rng.choice([1, 2, 5, 8, 16, 20]))
+        Hq = Hkv * hpk
+        L = int(rng.choice(edges)) if case % 2 == 0 else int(rng.integers(1, 9000))
+        bf16 = bool(case % 3)
+        q, g, k, v = sdpa_random_inputs(7000 + case, Hq, Hkv, d, L, bf16=bf16)
+        ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+        out = mfa.sdpa_cpu(L, Hq, Hkv, d, q, g, k, v)
+        tol = 1e-4 if bf16 else TOL_F32
+        assert rel_err(out, ref) <= tol, (case, d, Hq, Hkv, L, bf16, rel_err(out, ref))
+
+
 def test_config1_full_size(mfa, oracle):
     """The 4K f32 decode shape: 32 Q / 4 KV heads, d=128, L=4096, fp32."""
     Hq, Hkv, d, L = 32, 4, 128, 4096
