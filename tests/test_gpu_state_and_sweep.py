@@ -60,6 +60,32 @@ def test_prefill_attn_few_tokens_after_a_long_cache(mfa, oracle, bf16):
     assert rel_err(out, ref) <= (1e-4 if bf16 else TOL_F32)
 
 
+def test_prefill_attn_short_chunks_random_shapes(mfa, oracle):
+    """Seeded random short chunks behind caches of random length: the split-K path with per-row
+    causal limits under the default split planning, every head_dim, f32 and bf16 caches, ragged
+    row groups."""
+    rng = np.random.default_rng(77)
+    for case in range(12):
+        d = int(rng.choice([64, 128, 256]))
+        Hkv = int(rng.choice([1, 2, 4]))
+        Hq = Hkv * int(rng.choice([1, 3, 4, 8, 16]))
+        T = int(rng.integers(2, 13))
+        L0 = int(rng.choice([511, 2047, 2049, 4096, 6145])) if case % 2 else int(rng.integers(300, 9000))
+        bf16 = bool(case % 3)
+        k = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+        v = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+        if bf16:
+            k, v = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k, v))
+        q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+        g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+        ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+        with _full_ctx(mfa, Hq, Hkv, d, L0 + T, bf16=bf16) as c:
+            c.kv_import(0, k[:L0], v[:L0])
+            out = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+        err = rel_err(out, ref)
+        assert err <= (1e-4 if bf16 else TOL_F32), (case, d, Hq, Hkv, T, L0, bf16, err)
+
+
 @pytest.mark.parametrize("Hq,Hkv,d,T,L0,bf16", [(32, 2, 256, 70, 100, True), (8, 2, 64, 200, 0, False),
                                                 (32, 2, 256, 40, 9, False), (16, 4, 64, 130, 77, True),
                                                 (32, 4, 128, 1100, 50, True), (32, 16, 64, 2100, 0, True),
