@@ -124,6 +124,32 @@ def test_ctx_append_decode_and_split_invariance(mfa, oracle, bf16):
         assert np.array_equal(ke, kf) and np.array_equal(ve, vf)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_merge_of_several_hundred_splits(mfa, oracle, bf16):
+    """More splits than the 256 whose statistics the merge keeps in registers (the rest are read
+    in loops), and more than the 128 whose rows a thread requests up front: forced split counts
+    of 300, 512 and 1024 over a cache long enough to give every split a block."""
+    Hq, Hkv, d, L = 8, 1, 64, 17000
+    q, g, k, v = sdpa_random_inputs(71, Hq, Hkv, d, L, bf16=bf16)
+    kf = oracle.bf16_to_f32(k) if bf16 else k
+    vf = oracle.bf16_to_f32(v) if bf16 else v
+    ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+    from moeflux_amd import ffi
+    with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
+              head_dim=d, kv_capacity=L, kv_dtype=1 if bf16 else 0) as c:
+        c.kv_import(0, kf, vf)
+        base = c.sdpa_decode(0, q, g)
+        assert rel_err(base, ref) <= (1e-4 if bf16 else TOL_F32)
+        seen = set()
+        for ns in (300, 512, 1024):
+            c.set_num_splits(ns)
+            seen.add(c.lib.mfa_debug_num_splits(1 if bf16 else 0, Hq, Hkv, d, L, 256, ns))
+            out = c.sdpa_decode(0, q, g)
+            assert rel_err(out, ref) <= (1e-4 if bf16 else TOL_F32), ns
+            assert rel_err(out, base) <= 1e-5, ns
+        assert max(seen) > 256
+
+
 def test_config3_full_size_bf16(mfa, oracle):
     """The 32K bf16 decode shape (the headline workload): 32 Q / 2 KV heads, d=256, L=32768, bf16 K/V, via bulk import."""
     Hq, Hkv, d, L = 32, 2, 256, 32768
