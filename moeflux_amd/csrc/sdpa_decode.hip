@@ -306,12 +306,64 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     }
 }
 
+// The merge for few splits (at most NS = 8 or 16, what a launch over many layers or row groups
+// ends up with): one wave per 64 outputs of a (token, head) row, four such units per workgroup,
+// no LDS and no barrier (the 12-layer sweep's merge: 5.0 -> 3 us; no gain from 32 splits on).  Lane s holds split s's (max, sum); a
+// lane's output is the weighted sum of one float per split, all requested before the first use.
+template <int NS>
+__global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
+    const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
+    int Hq, int nhg, int D, int n_units, const float *__restrict__ gate, float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (unit >= n_units) return;   // whole waves; there is no barrier below
+    const int per_row = D / 64, bx = unit / per_row, by = unit % per_row;
+    const int h = bx % Hq, tok = bx / Hq;
+    const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
+    const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
+    const float *ml = part_ml + pid0 * 32 + n;
+    const int d = by * 64 + lane;
+    const int sl = lane < nsplit ? lane : nsplit - 1;
+    const float m_in = ml[(size_t)sl * 32], l_in = ml[(size_t)sl * 32 + 16];
+    float rows[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) rows[s] = part_o[((pid0 + (s < nsplit ? s : nsplit - 1)) * 16 + n) * D + d];
+    const float gt_in = gate ? gate[(size_t)bx * D + d] : 0.f;
+
+    const float ms = lane < nsplit ? m_in : neg_inf();
+    const float M = wave_max(ms);
+    const float w = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
+    const float den = group_sum<64>(w * (lane < nsplit ? l_in : 0.f));
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const float ws = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s));
+        acc += ws * rows[s];   // ws is 0 for s >= nsplit
+    }
+    const float gt = gate ? 1.0f / (1.0f + expf(-gt_in)) : 1.0f;
+    out[(size_t)bx * D + d] = (acc / den) * gt;
+}
+
+static void launch_merge_kernels(hipStream_t stream, const float *part_o, const float *part_ml, int splits, int hpk,
+                                 int Hq, int nhg, int D, int n_tok, const float *gate, float *out) {
+    const int n_units = n_tok * Hq * (D / 64);
+    const dim3 few((n_units + 3) / 4);
+    if (splits <= 8)
+        hipLaunchKernelGGL((sdpa_merge_few_kernel<8>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
+                           n_units, gate, out);
+    else if (splits <= 16)
+        hipLaunchKernelGGL((sdpa_merge_few_kernel<16>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
+                           n_units, gate, out);
+    else
+        hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, part_o, part_ml, splits, hpk,
+                           Hq, nhg, D, gate, out);
+}
+
 int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,
                       int n_tok, const float *gate, float *out) {
     if (splits < 1 || splits > kMaxSplits || D % 64 != 0)
         return fail(MFA_ERR_INVALID, "merge: %d splits (1..%d), width %d (multiple of 64)", splits, kMaxSplits, D);
-    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, ws.part_o, ws.part_ml,
-                       splits, hpk, Hq, nhg, D, gate, out);
+    launch_merge_kernels(stream, ws.part_o, ws.part_ml, splits, hpk, Hq, nhg, D, n_tok, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }
@@ -435,8 +487,7 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
 #undef MFA_LAUNCH
     MFA_HIP(hipGetLastError());
     if (partial_only) return MFA_OK;
-    hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, ws.part_o,
-                       ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, gate, out);
+    launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, n_tok, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }
