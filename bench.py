@@ -378,6 +378,88 @@ def bench_matvec(steps, warmup, seed):
     return res
 
 
+def bench_prologue(steps, warmup, seed):
+    """What precedes the attention core in a full-attention layer, at the headline shape (32 Q /
+    2 KV heads, head_dim 256, bf16 cache holding 32768 positions): the prologue alone (q/gate
+    split, per-head norms, rotation, cache append - one launch) and the whole layer step
+    (prologue + split-K attention + merge over the grown cache, mfa_full_attn_step_dev)."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    from oracle import cref
+    lib = ffi.load()
+    Hq, Hkv, d, L = 32, 2, 256, 32768
+    n = 2 * (steps + warmup) + 8
+    ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                     kv_capacity=L + n, kv_dtype=ffi.KV_BF16))
+    rng = np.random.default_rng(seed)
+    kv = cref.f32_to_bf16(rng.standard_normal((L, Hkv * d), dtype=np.float32))
+    ctx.kv_import(0, kv, kv)
+    w = cref.f32_to_bf16(np.ones(d, np.float32))
+    ctx.set_full_weights(0, w, w)
+    qp = DeviceArray.from_host(rng.standard_normal(2 * Hq * d).astype(np.float32))
+    k = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
+    v = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
+    q, g, o = (DeviceArray((Hq * d,), np.float32, zero=True) for _ in range(3))
+    pos = [L]
+
+    def pro(i):
+        if lib.mfa_attn_prologue_dev(ctx.h, 0, pos[0], qp.ptr, k.ptr, v.ptr, q.ptr, g.ptr) != 0:
+            raise RuntimeError(ffi.last_error())
+        pos[0] += 1
+
+    def full(i):
+        if lib.mfa_full_attn_step_dev(ctx.h, 0, pos[0], qp.ptr, k.ptr, v.ptr, o.ptr) != 0:
+            raise RuntimeError(ffi.last_error())
+        pos[0] += 1
+
+    _, pro_ms = _timed(ctx, lib, pro, steps, warmup)
+    _, full_ms = _timed(ctx, lib, full, steps, warmup)
+    alg = 2 * Hq * d * 4 + 2 * Hkv * d * 4 + 2 * Hq * d * 4 + 2 * Hkv * d * 2
+    res = {"shape": "32 Q / 2 KV heads, head_dim 256, bf16 cache, kv_len 32768 and growing",
+           "prologue_us_per_call": pro_ms * 1e3, "prologue_algorithmic_bytes": alg,
+           "full_attn_step_us_per_call": full_ms * 1e3, "launches_per_full_step": 3}
+    ctx.close()
+    for a in (qp, k, v, q, g, o):
+        a.free()
+    return res
+
+
+def bench_snapshot(seed):
+    """The 'MFLX' snapshot of a 48-layer hybrid stack (36 DeltaNet layers, 12 full-attention layers
+    with 2048 cached positions each): bytes, and the time to save it to and load it from host
+    memory (device reads and writes, conversion from and to the tiled cache, PCIe both ways)."""
+    from moeflux_amd import Config, Ctx, ffi
+    from oracle import cref
+    lib = ffi.load()
+    NL, Hq, Hkv, d, L = 48, 32, 2, 256, 2048
+    ctx = Ctx(Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                     kv_capacity=L, kv_dtype=ffi.KV_BF16, linear_num_k_heads=16, linear_num_v_heads=32))
+    rng = np.random.default_rng(seed)
+    kv = cref.f32_to_bf16(rng.standard_normal((L, Hkv * d), dtype=np.float32))
+    for i in range(NL):
+        if (i + 1) % 4 == 0:
+            ctx.kv_import(i, kv, kv)
+    size = ctx.state_size()
+    buf = np.empty(size, np.uint8)
+    p = buf.ctypes.data_as(C.c_void_p)
+    times = {"save": [], "load": []}
+    for _ in range(3):
+        t0 = time.perf_counter()
+        nbytes = lib.mfa_state_save(ctx.h, p, size)
+        times["save"].append(time.perf_counter() - t0)
+        if nbytes != size:
+            raise RuntimeError("mfa_state_save: %d of %d bytes" % (nbytes, size))
+        t0 = time.perf_counter()
+        if lib.mfa_state_load(ctx.h, p, size) != 0:
+            raise RuntimeError(ffi.last_error())
+        lib.mfa_sync(ctx.h)
+        times["load"].append(time.perf_counter() - t0)
+    ctx.close()
+    return {"layers": NL, "kv_len": L, "bytes": size, "save_ms": min(times["save"]) * 1e3,
+            "load_ms": min(times["load"]) * 1e3, "save_gbps": size / min(times["save"]) / 1e9,
+            "load_gbps": size / min(times["load"]) / 1e9}
+
+
 def bench_mla(steps, warmup, seed, lens=(4096, 32768)):
     """Attention of one token over a latent cache at the MLA variants' shape (128 heads,
     kv_lora_rank 512, qk_rope_head_dim 64; variants.rs), f32 caches, cache sets rotated."""
@@ -500,7 +582,7 @@ def main():
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
     ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
     ap.add_argument("--f4-len", type=int, default=0, help="one cache length for --only f4 (default: 4096 and 32768)")
-    ap.add_argument("--only", choices=["c4", "c5", "f3", "f4"], default=None,
+    ap.add_argument("--only", choices=["c4", "c5", "f1", "f2", "f3", "f4"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -513,6 +595,12 @@ def main():
 
     if a.only == "c4":
         print(json.dumps({f"c4_prefill_chunk_{a.tokens}": bench_prefill(a.steps, a.warmup, 0xC0FFEE + 4, a.tokens)}))
+        return
+    if a.only == "f1":
+        print(json.dumps({"f1_attention_prologue": bench_prologue(a.steps, a.warmup, 0xC0FFEE + 8)}))
+        return
+    if a.only == "f2":
+        print(json.dumps({"f2_state_snapshot": bench_snapshot(0xC0FFEE + 9)}))
         return
     if a.only == "f3":
         print(json.dumps({"f3_projection_matvecs": bench_matvec(a.steps, a.warmup, 0xC0FFEE + 6)}))
@@ -557,6 +645,8 @@ def main():
                                                     0xC0FFEE + 2)
         extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
         extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
+        extra["f1_attention_prologue"] = bench_prologue(max(50, a.steps // 4), 10, 0xC0FFEE + 8)
+        extra["f2_state_snapshot"] = bench_snapshot(0xC0FFEE + 9)
         extra["f3_projection_matvecs"] = bench_matvec(a.steps // 2, a.warmup, 0xC0FFEE + 6)
         extra["f4_mla_folded_sdpa"] = bench_mla(max(20, a.steps // 8), 5, 0xC0FFEE + 7)
         if not a.no_cpu:
