@@ -207,3 +207,17 @@ def test_chunk_at_the_a17b_head_counts(mfa):
         out = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
         _, ssm = c.linear_state_export(0)
     assert rel_err(out, ref_out) <= TOL_F32 and rel_err(ssm, ref_ssm) <= TOL_F32
+
+
+def test_prompt_longer_than_one_segment(mfa):
+    """A prompt of more than 4096 tokens goes through the chunk kernels in 4096-token segments; the
+    ring and the state carry from one segment to the next as they do between calls."""
+    case = GdnCase(8, 2, 4, 64, 64, T=4096 + 70)
+    ref_out, ref_conv, ref_ssm = case.oracle()
+    with _ctx(mfa, case) as c:
+        c.linear_state_import(0, case.conv_state, case.ssm_state)
+        out = c.prefill_gdn(0, case.qkv, case.z, case.alpha, case.beta)
+        conv, ssm = c.linear_state_export(0)
+    assert rel_err(out, ref_out) <= TOL_F32 and rel_err(ssm, ref_ssm) <= TOL_F32
+    assert rel_err(out[4090:], ref_out[4090:]) <= 5e-5
+    assert np.array_equal(conv.reshape(-1), ref_conv)

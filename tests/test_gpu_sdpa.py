@@ -161,3 +161,16 @@ def test_config3_full_size_bf16(mfa, oracle):
         out = c.sdpa_decode(0, q, g)
     assert rel_err(out, ref) <= TOL_BF16
     assert rel_err(out, ref) <= 1e-4
+
+
+def test_cache_of_131072_positions_bf16(mfa, oracle):
+    """Four times the 32K decode shape's length: 4096 blocks per kv head, 268 MB per layer, four passes
+    per workgroup; the byte offsets of the last blocks pass 2^27."""
+    Hq, Hkv, d, L = 32, 2, 256, 131072
+    q, g, k, v = sdpa_random_inputs(0xC0FFEE + 13, Hq, Hkv, d, L, bf16=True)
+    ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+    with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
+              head_dim=d, kv_capacity=L, kv_dtype=1) as c:
+        c.kv_import(0, k, v)
+        out = c.sdpa_decode(0, q, g)
+    assert rel_err(out, ref) <= 1e-4

@@ -89,7 +89,8 @@ def test_prefill_attn_short_chunks_random_shapes(mfa, oracle):
 @pytest.mark.parametrize("Hq,Hkv,d,T,L0,bf16", [(32, 2, 256, 70, 100, True), (8, 2, 64, 200, 0, False),
                                                 (32, 2, 256, 40, 9, False), (16, 4, 64, 130, 77, True),
                                                 (32, 4, 128, 1100, 50, True), (32, 16, 64, 2100, 0, True),
-                                                (32, 16, 64, 2050, 3, False)])
+                                                (32, 16, 64, 2050, 3, False), (4, 1, 64, 4200, 100, True),
+                                                (2, 1, 128, 4100, 0, False)])
 def test_prefill_attn_shapes(mfa, oracle, Hq, Hkv, d, T, L0, bf16):
     """The chunk kernel (one wave per 16-row group, K/V blocks staged in LDS) over head
     dims, group sizes, ragged row counts and one or two row groups per wave."""
