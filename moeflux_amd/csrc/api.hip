@@ -259,16 +259,8 @@ static int truncate_full(Ctx *c, FullLayer &f, int32_t new_len) {
     return MFA_OK;
 }
 
-// The split-K workspace is sized for decode at create time; a prompt chunk has n_tok times
-// the rows and grows it on first use.
-// `layers` > 1 sizes it for one launch over that many layers (layers * Hkv kv heads).
-static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
-    const mfa_config &g = c->cfg;
-    const int Hq = g.num_attn_heads * layers, Hkv = g.num_kv_heads * layers;
-    int splits = sdpa_pick_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
-    if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
-    const size_t need_o = sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok);
-    const size_t need_ml = sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok);
+// Grows the split-K workspace to at least the given element counts (never shrinks it).
+static int ensure_workspace_elems(Ctx *c, size_t need_o, size_t need_ml) {
     if (need_o <= c->part_o_elems && need_ml <= c->part_ml_elems) return MFA_OK;
     MFA_HIP(hipStreamSynchronize(c->stream));
     if (need_o > c->part_o_elems) {
@@ -286,6 +278,18 @@ static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
         c->part_ml_elems = need_ml;
     }
     return MFA_OK;
+}
+
+// The split-K workspace is sized for decode at create time; a prompt chunk has n_tok times
+// the rows and grows it on first use.
+// `layers` > 1 sizes it for one launch over that many layers (layers * Hkv kv heads).
+static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
+    const mfa_config &g = c->cfg;
+    const int Hq = g.num_attn_heads * layers, Hkv = g.num_kv_heads * layers;
+    int splits = sdpa_pick_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
+    if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
+    return ensure_workspace_elems(c, sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok),
+                                  sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok));
 }
 
 // n_tok tokens whose K/V rows are already in the cache (the last n_tok positions).
@@ -450,6 +454,8 @@ int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits) {
     if (!c) return fail(MFA_ERR_INVALID, "NULL context");
     if (num_splits < 0) return fail(MFA_ERR_INVALID, "num_splits must be >= 0");
     c->forced_splits = num_splits;
+    // a forced count is used as given, so the workspace must hold it at any cache length
+    if (num_splits > 0 && !c->full.empty()) MFA_TRY(ensure_workspace(c, 1, c->cfg.kv_capacity));
     return MFA_OK;
 }
 
@@ -764,26 +770,6 @@ int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on) {
 }
 
 /* ---- attention over a latent cache -------------------------------------------------- */
-
-static int ensure_workspace_elems(Ctx *c, size_t need_o, size_t need_ml) {
-    if (need_o <= c->part_o_elems && need_ml <= c->part_ml_elems) return MFA_OK;
-    MFA_HIP(hipStreamSynchronize(c->stream));
-    if (need_o > c->part_o_elems) {
-        if (c->part_o) MFA_HIP(hipFree(c->part_o));
-        c->part_o = nullptr;
-        c->part_o_elems = 0;
-        MFA_HIP(hipMalloc((void **)&c->part_o, need_o * sizeof(float)));
-        c->part_o_elems = need_o;
-    }
-    if (need_ml > c->part_ml_elems) {
-        if (c->part_ml) MFA_HIP(hipFree(c->part_ml));
-        c->part_ml = nullptr;
-        c->part_ml_elems = 0;
-        MFA_HIP(hipMalloc((void **)&c->part_ml, need_ml * sizeof(float)));
-        c->part_ml_elems = need_ml;
-    }
-    return MFA_OK;
-}
 
 static int mla_check(int32_t H, int32_t R, int32_t P, int32_t L) {
     if (H <= 0 || R <= 0 || P <= 0) return fail(MFA_ERR_INVALID, "non-positive shape");

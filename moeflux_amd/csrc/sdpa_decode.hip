@@ -460,13 +460,14 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
         return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld for %d tokens)", (long long)kv_len, n_tok);
     const int hpk = Hq / Hkv;
     SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
-    // never exceed the workspace
-    while (plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
+    // never exceed the workspace: a split count shrinks to fit, except one forced for a single
+    // token, which is used as given or refused
+    while ((forced_splits <= 0 || n_tok > 1) && plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
                                sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems))
         plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
     if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
         sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems)
-        return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small");
+        return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
     if (plan.nhg > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
     // scores are produced in log2 units: q is pre-multiplied by (1/sqrt(D)) * log2(e)
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
