@@ -35,6 +35,24 @@ def test_every_declared_symbol_is_exported_and_bound():
     assert sorted(ffi.SIGNATURES) == syms, "ctypes table and header disagree"
 
 
+def test_rust_view_declares_every_entry_point_with_the_headers_parameter_count():
+    """moeflux_amd/rust/ffi.rs cannot be compiled here; names, parameter counts and the
+    pointer/scalar kind of every parameter are held to the header instead."""
+    plain = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    plain = re.sub(r"//[^\n]*", "", plain)
+    c_protos = {m.group(1): m.group(2) for m in re.finditer(r"\b(mfa_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", plain)}
+    rust = open(os.path.join(ROOT, "moeflux_amd", "rust", "ffi.rs")).read()
+    r_protos = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (mfa_[a-z0-9_]+)\(([^;]*?)\)\s*(?:->[^;]*)?;", rust, flags=re.S)}
+    assert sorted(r_protos) == declared_symbols()
+    for name, args in c_protos.items():
+        c_args = [] if args.strip() in ("", "void") else [a.strip() for a in args.split(",")]
+        r_args = [a.strip() for a in r_protos[name].split(",") if a.strip()]
+        assert len(c_args) == len(r_args), name
+        for ca, ra in zip(c_args, r_args):
+            assert ("*" in ca) == ("*" in ra), (name, ca, ra)
+            assert ("const" in ca.split("*")[0].split()) == ("*const" in ra) if "*" in ca else True, (name, ca, ra)
+
+
 def test_header_cites_the_reference_for_every_entry_point():
     # each declaration is preceded by a comment naming a reference file or saying it has none
     for name in declared_symbols():
