@@ -427,7 +427,8 @@ def bench_prologue(steps, warmup, seed):
 def bench_snapshot(seed):
     """The 'MFLX' snapshot of a 48-layer hybrid stack (36 DeltaNet layers, 12 full-attention layers
     with 2048 cached positions each): bytes, and the time to save it to and load it from host
-    memory (device reads and writes, conversion from and to the tiled cache, PCIe both ways)."""
+    memory (device reads and writes, conversion from and to the tiled cache, PCIe both ways);
+    beside it the same state stored and restored as a device-resident checkpoint."""
     from moeflux_amd import Config, Ctx, ffi
     from oracle import cref
     lib = ffi.load()
@@ -454,10 +455,23 @@ def bench_snapshot(seed):
             raise RuntimeError(ffi.last_error())
         lib.mfa_sync(ctx.h)
         times["load"].append(time.perf_counter() - t0)
+    # the same state as a checkpoint kept on the device (mfa_checkpoint_pos / mfa_restore_to)
+    times["checkpoint"], times["restore"] = [], []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        if lib.mfa_checkpoint_pos(ctx.h, L) != 0:
+            raise RuntimeError(ffi.last_error())
+        times["checkpoint"].append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        if lib.mfa_restore_to(ctx.h, L) != 0:
+            raise RuntimeError(ffi.last_error())
+        times["restore"].append(time.perf_counter() - t0)
     ctx.close()
     return {"layers": NL, "kv_len": L, "bytes": size, "save_ms": min(times["save"]) * 1e3,
             "load_ms": min(times["load"]) * 1e3, "save_gbps": size / min(times["save"]) / 1e9,
-            "load_gbps": size / min(times["load"]) / 1e9}
+            "load_gbps": size / min(times["load"]) / 1e9,
+            "device_checkpoint_ms": min(times["checkpoint"]) * 1e3,
+            "device_restore_ms": min(times["restore"]) * 1e3}
 
 
 def bench_mla(steps, warmup, seed, lens=(4096, 32768)):

@@ -43,6 +43,7 @@ typedef struct mfa_ctx mfa_ctx;
 #define MFA_ERR_LAYER (-4)    /* layer index out of range or of the other kind */
 #define MFA_ERR_HIP (-5)      /* a HIP runtime call failed; see mfa_last_error_string() */
 #define MFA_ERR_STATE (-6)    /* snapshot does not match this context (state_snapshot.rs preflight) */
+#define MFA_ERR_NO_CHECKPOINT (-7) /* mfa_restore_to: nothing stored at that position (CheckpointError::NoCheckpoint, riir/mod.rs:111-124) */
 
 #define MFA_KV_F32 0
 #define MFA_KV_BF16 1
@@ -282,7 +283,7 @@ int mfa_set_sweep_per_layer(mfa_ctx *ctx, int32_t on);
 /* ---- state operations ------------------------------------------------------ */
 
 /* memory_clear (riir/mod.rs:1950-1969; state.rs clear_all): KV lengths to 0,
- * caches zeroed, conv and recurrent state zeroed. */
+ * caches zeroed, conv and recurrent state zeroed, checkpoints dropped. */
 int mfa_reset(mfa_ctx *ctx);
 /* memory_seq_rm (state.rs:431-455): every KV cache keeps positions
  * [0, min(max(p0,0), p1<0 ? len : min(p1,len))) and the dropped rows are
@@ -319,6 +320,26 @@ int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state
 int64_t mfa_state_size(mfa_ctx *ctx);
 int64_t mfa_state_save(mfa_ctx *ctx, uint8_t *buf, int64_t buf_len);
 int mfa_state_load(mfa_ctx *ctx, const uint8_t *buf, int64_t buf_len);
+
+/* Checkpoints keyed by sequence position, for rewinding to a prompt-cache
+ * breakpoint without prefilling again (RsCtx::checkpoint_pos riir/mod.rs:2015-2061,
+ * restore_to :2072-2087, set_max_checkpoints :2094-2096, checkpoint_count :2098-2100;
+ * tests/checkpoint_restore.rs).  The reference keeps state_save buffers on the host;
+ * here a checkpoint is a device-resident copy of the same state (every KV cache up to
+ * its length, every conv state and recurrent state) and costs device memory of about
+ * mfa_state_size bytes (half that for the KV part of a bf16 cache).
+ * mfa_checkpoint_pos stores the current state under `pos`; a checkpoint already at
+ * `pos` is replaced and becomes the newest.  Beyond the cap (default 4) the oldest is
+ * dropped, never position 0 nor the one just stored.
+ * mfa_restore_to brings back exactly the stored state, then drops every checkpoint
+ * at a position > pos; MFA_ERR_NO_CHECKPOINT, with nothing changed, when there is none
+ * at `pos`.  mfa_set_max_checkpoints takes effect at the next store.  mfa_reset drops
+ * all checkpoints (memory_clear, riir/mod.rs:1965-1968); mfa_truncate and
+ * mfa_state_load leave them, as in the reference.  Call at token boundaries only. */
+int mfa_checkpoint_pos(mfa_ctx *ctx, int32_t pos);
+int mfa_restore_to(mfa_ctx *ctx, int32_t pos);
+int mfa_set_max_checkpoints(mfa_ctx *ctx, int32_t n);
+int32_t mfa_checkpoint_count(mfa_ctx *ctx);
 
 /* ---- timing ---------------------------------------------------------------- */
 

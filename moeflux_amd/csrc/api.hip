@@ -78,6 +78,7 @@ static void destroy(Ctx *c) {
     if (!c) return;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
+    drop_checkpoints(c);
     for (void *p : c->slabs)
         if (p) (void)hipFree(p);
     if (c->part_o) (void)hipFree(c->part_o);
@@ -886,6 +887,7 @@ int mfa_reset(mfa_ctx *ctx) {
     for (auto &f : c->full) MFA_TRY(truncate_full(c, f, 0));
     for (auto &l : c->lin) MFA_TRY(reset_linear(c, l));
     MFA_HIP(hipStreamSynchronize(c->stream));
+    drop_checkpoints(c);  // keyed by position: a full clear invalidates every key (riir/mod.rs:1965-1968)
     return MFA_OK;
 }
 

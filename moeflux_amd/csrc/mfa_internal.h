@@ -118,6 +118,15 @@ struct LinearLayer {
     LinearWeights w;
 };
 
+// The state at one sequence position, kept on the device (checkpoint.hip).
+struct Checkpoint {
+    int32_t pos = 0;
+    char *buf = nullptr;              // one allocation: K prefixes, V prefixes, rings, recurrent states
+    size_t bytes = 0;
+    std::vector<int32_t> full_len;    // cache length of every full-attention layer
+    std::vector<int64_t> lin_step;    // ring position of every linear layer
+};
+
 struct Ctx {
     mfa_config cfg{};
     int device = 0;
@@ -150,6 +159,9 @@ struct Ctx {
     float *pinned = nullptr;
     size_t pinned_elems = 0;
     int num_cus = 256;
+    // checkpoints by position, least recently stored first (checkpoint.hip)
+    std::vector<Checkpoint> checkpoints;
+    size_t max_checkpoints = 4;       // DEFAULT_MAX_CHECKPOINTS, riir/mod.rs:105-109
 
     int conv_dim() const {
         return 2 * cfg.linear_num_k_heads * cfg.linear_key_dim +
@@ -236,6 +248,9 @@ int launch_kv_zero(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plan
                    int64_t pos0, int64_t pos1, void *k_tiled, void *v_tiled);
 
 int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+
+// checkpoint.hip
+void drop_checkpoints(Ctx *c);   // frees every stored checkpoint (reset, destroy)
 
 // attn_kernels.hip (the four reference kernels, one launch each)
 int launch_attn_scores(hipStream_t s, int Hq, int Hkv, int D, int L, int stride, const float *q,

@@ -268,6 +268,20 @@ class Ctx:
         buf = np.frombuffer(blob, dtype=np.uint8)
         _chk(self.lib.mfa_state_load(self.h, _p(buf) if buf.size else None, buf.size), "mfa_state_load")
 
+    # checkpoints by position (riir/mod.rs:2015-2100)
+    def checkpoint_pos(self, pos: int):
+        _chk(self.lib.mfa_checkpoint_pos(self.h, pos), "mfa_checkpoint_pos")
+
+    def restore_to(self, pos: int):
+        """Raises MfaError with code ffi.ERR_NO_CHECKPOINT when nothing is stored at `pos`."""
+        _chk(self.lib.mfa_restore_to(self.h, pos), "mfa_restore_to")
+
+    def set_max_checkpoints(self, n: int):
+        _chk(self.lib.mfa_set_max_checkpoints(self.h, n), "mfa_set_max_checkpoints")
+
+    def checkpoint_count(self) -> int:
+        return _chk(self.lib.mfa_checkpoint_count(self.h), "mfa_checkpoint_count")
+
     def sync(self):
         _chk(self.lib.mfa_sync(self.h), "mfa_sync")
 

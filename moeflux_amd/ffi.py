@@ -12,7 +12,7 @@ import os
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
                          "libmoeflux_attn_hip.so")
 
-OK, ERR_INVALID, ERR_SHAPE, ERR_OVERFLOW, ERR_LAYER, ERR_HIP, ERR_STATE = 0, -1, -2, -3, -4, -5, -6
+OK, ERR_INVALID, ERR_SHAPE, ERR_OVERFLOW, ERR_LAYER, ERR_HIP, ERR_STATE, ERR_NO_CHECKPOINT = 0, -1, -2, -3, -4, -5, -6, -7
 KV_F32, KV_BF16 = 0, 1
 
 i32, f32, vp, u16p, f32p = C.c_int32, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p
@@ -71,6 +71,10 @@ SIGNATURES = {
     "mfa_state_size": (C.c_int64, [vp]),
     "mfa_state_save": (C.c_int64, [vp, vp, C.c_int64]),
     "mfa_state_load": (C.c_int, [vp, vp, C.c_int64]),
+    "mfa_checkpoint_pos": (C.c_int, [vp, i32]),
+    "mfa_restore_to": (C.c_int, [vp, i32]),
+    "mfa_set_max_checkpoints": (C.c_int, [vp, i32]),
+    "mfa_checkpoint_count": (i32, [vp]),
     "mfa_set_sweep_per_layer": (C.c_int, [vp, C.c_int32]),
     "mfa_token_sweep_dev": (C.c_int, [vp, f32p, f32p, f32p, f32p, f32p, f32p, f32p, f32p]),
     "mfa_reset": (C.c_int, [vp]),

@@ -16,7 +16,7 @@ fn main() {
         .arg("-I").arg(root.join("include")).arg("-I").arg(&csrc);
     for f in [
         "api.hip", "kv_cache.hip", "sdpa_decode.hip", "sdpa_prefill.hip", "attn_kernels.hip", "gdn.hip",
-        "gdn_chunk.hip", "gdn_wy.hip", "attn_prologue.hip", "snapshot.hip", "dequant_matvec.hip", "mla_sdpa.hip",
+        "gdn_chunk.hip", "gdn_wy.hip", "attn_prologue.hip", "snapshot.hip", "dequant_matvec.hip", "mla_sdpa.hip", "checkpoint.hip",
     ] {
         println!("cargo:rerun-if-changed=csrc/{f}");
         cmd.arg(csrc.join(f));

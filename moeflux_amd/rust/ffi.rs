@@ -83,6 +83,11 @@ extern "C" {
     pub fn mfa_state_size(ctx: *mut mfa_ctx) -> i64;
     pub fn mfa_state_save(ctx: *mut mfa_ctx, buf: *mut u8, buf_len: i64) -> i64;
     pub fn mfa_state_load(ctx: *mut mfa_ctx, buf: *const u8, buf_len: i64) -> c_int;
+    // checkpoints by sequence position, kept on the device
+    pub fn mfa_checkpoint_pos(ctx: *mut mfa_ctx, pos: i32) -> c_int;
+    pub fn mfa_restore_to(ctx: *mut mfa_ctx, pos: i32) -> c_int;
+    pub fn mfa_set_max_checkpoints(ctx: *mut mfa_ctx, n: i32) -> c_int;
+    pub fn mfa_checkpoint_count(ctx: *mut mfa_ctx) -> i32;
 
     // host-pointer forms of the layer step and the bulk bf16 import
     pub fn mfa_attn_prologue(ctx: *mut mfa_ctx, layer: i32, pos: i32, q_proj_out: *const f32,
