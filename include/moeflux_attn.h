@@ -223,6 +223,18 @@ int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_
                        const float *k, const float *v, float *out);
 int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
                            const float *k_dev, const float *v_dev, float *out_dev);
+/* The same for a chunk of T prompt tokens at positions pos0 .. pos0+T-1 (the token
+ * loop of eval_prompt, riir/mod.rs:1196-1214, over full_attn_layer_forward): every
+ * token's q and k are normed and rotated at its own position, the T rows are
+ * appended, and row t attends to the cache up to and including itself.  Same
+ * results as T calls of mfa_full_attn_step.  q_proj_out: [T][Hq][2*head_dim],
+ * k, v: [T][num_kv_heads*head_dim], out: [T][Hq*head_dim].  Nothing is appended
+ * when the call fails (MFA_ERR_OVERFLOW when the chunk does not fit). */
+int mfa_prefill_full_attn(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t T,
+                          const float *q_proj_out, const float *k, const float *v, float *out);
+int mfa_prefill_full_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t T,
+                              const float *q_proj_out_dev, const float *k_dev,
+                              const float *v_dev, float *out_dev);
 
 /* A chunk of T prompt tokens on one full-attention layer.  The reference has
  * no batched prefill: eval_prompt is a token loop (riir/mod.rs:1196-1214); the

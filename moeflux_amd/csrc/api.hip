@@ -85,6 +85,7 @@ static void destroy(Ctx *c) {
     if (c->part_ml) (void)hipFree(c->part_ml);
     if (c->stage) (void)hipFree(c->stage);
     if (c->gdn_scratch) (void)hipFree(c->gdn_scratch);
+    if (c->qg_chunk) (void)hipFree(c->qg_chunk);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -540,15 +541,16 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
     return d2h_sync(c, out, c->stage + 2 * qd, qd * 4);
 }
 
+// n_tok tokens at positions pos .. pos + n_tok - 1, appended at the end of the layer's cache.
 static int prologue_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_proj, const float *k, const float *v,
-                        float *q_out, float *gate_out) {
+                        float *q_out, float *gate_out, int32_t n_tok = 1) {
     if (!f->norms_set) return fail(MFA_ERR_INVALID, "q/k norm weights not set (mfa_set_full_weights)");
-    if ((int64_t)f->len + 1 > c->cfg.kv_capacity)
-        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + 1 > capacity %d", f->len, c->cfg.kv_capacity);
+    if ((int64_t)f->len + n_tok > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %d > capacity %d", f->len, n_tok, c->cfg.kv_capacity);
     MFA_TRY(launch_attn_prologue(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads, c->cfg.num_kv_heads,
-                                 c->cfg.head_dim, c->rotary_dim, c->cfg.rms_norm_eps, pos, f->len, c->plane_elems,
+                                 c->cfg.head_dim, c->rotary_dim, c->cfg.rms_norm_eps, n_tok, pos, f->len, c->plane_elems,
                                  f->q_norm, f->k_norm, c->inv_freq, q_proj, k, v, q_out, gate_out, f->k, f->v));
-    f->len += 1;
+    f->len += n_tok;
     return MFA_OK;
 }
 
@@ -605,6 +607,56 @@ int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_
     MFA_TRY(prologue_dev(c, f, pos, qp, kk, vv, c->qg_stage, c->qg_stage + qd));
     MFA_TRY(sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, oo));
     return d2h_sync(c, out, oo, qd * 4);
+}
+
+int mfa_prefill_full_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t T, const float *q_proj_out_dev,
+                              const float *k_dev, const float *v_dev, float *out_dev) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out_dev || !k_dev || !v_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    // everything that can fail is checked before the first token is appended
+    if (!f->norms_set) return fail(MFA_ERR_INVALID, "q/k norm weights not set (mfa_set_full_weights)");
+    if (pos0 < 0 || (int64_t)pos0 + T - 1 > INT32_MAX)
+        return fail(MFA_ERR_INVALID, "positions %d .. %lld out of range", pos0, (long long)pos0 + T - 1);
+    if ((int64_t)f->len + T > c->cfg.kv_capacity)
+        return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %d > capacity %d", f->len, T, c->cfg.kv_capacity);
+    const size_t qd = (size_t)c->q_dim() * T;
+    if (2 * qd > c->qg_chunk_elems) {
+        MFA_HIP(hipStreamSynchronize(c->stream));
+        if (c->qg_chunk) MFA_HIP(hipFree(c->qg_chunk));
+        c->qg_chunk = nullptr;
+        c->qg_chunk_elems = 0;
+        MFA_HIP(hipMalloc((void **)&c->qg_chunk, 2 * qd * sizeof(float)));
+        c->qg_chunk_elems = 2 * qd;
+    }
+    // the whole chunk is normed, rotated and appended, then one causal pass: row t sees positions [0, len0 + t]
+    const int kSeg = 32768;   // tokens per prologue launch (the grid's second dimension holds 65535)
+    for (int32_t off = 0; off < T; off += kSeg) {
+        const int32_t n = T - off < kSeg ? T - off : kSeg;
+        MFA_TRY(prologue_dev(c, f, pos0 + off, q_proj_out_dev + (size_t)off * 2 * c->q_dim(),
+                             k_dev + (size_t)off * c->kv_dim(), v_dev + (size_t)off * c->kv_dim(),
+                             c->qg_chunk + (size_t)off * c->q_dim(), c->qg_chunk + qd + (size_t)off * c->q_dim(), n));
+    }
+    return sdpa_dev(c, f, T, c->qg_chunk, c->qg_chunk + qd, out_dev);
+}
+
+int mfa_prefill_full_attn(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t T, const float *q_proj_out,
+                          const float *k, const float *v, float *out) {
+    Ctx *c = as_ctx(ctx);
+    FullLayer *f;
+    MFA_TRY(full_layer(c, layer, &f));
+    if (!q_proj_out || !k || !v || !out) return fail(MFA_ERR_INVALID, "NULL argument");
+    if (T <= 0) return fail(MFA_ERR_INVALID, "T must be > 0 (got %d)", T);
+    const size_t qd = (size_t)c->q_dim() * T, kvd = (size_t)c->kv_dim() * T;
+    MFA_TRY(ensure_stage(c, 3 * qd + 2 * kvd));
+    float *qp = c->stage, *dk = qp + 2 * qd, *dv = dk + kvd, *dout = dv + kvd;
+    MFA_TRY(h2d(c, qp, q_proj_out, 2 * qd * 4));
+    MFA_TRY(h2d(c, dk, k, kvd * 4));
+    MFA_TRY(h2d(c, dv, v, kvd * 4));
+    MFA_TRY(mfa_prefill_full_attn_dev(ctx, layer, pos0, T, qp, dk, dv, dout));
+    return d2h_sync(c, out, dout, qd * 4);
 }
 
 int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_dev,

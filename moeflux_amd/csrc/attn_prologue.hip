@@ -18,12 +18,14 @@ template <typename KV> __device__ inline KV to_kv(float x);
 template <> __device__ inline float to_kv<float>(float x) { return x; }
 template <> __device__ inline uint16_t to_kv<uint16_t>(float x) { return f32_to_bf16_bits(x); }
 
-// grid Hq + 2*Hkv workgroups of D threads (D = 64, 128 or 256):
+// grid (Hq + 2*Hkv, n_tok) workgroups of D threads (D = 64, 128 or 256); along x:
 //   [0, Hq)           q head: split off the gate, norm, rotate
 //   [Hq, Hq+Hkv)      k head: norm, rotate, store at cache position `cache_pos`
 //   [Hq+Hkv, Hq+2Hkv) v head: store at cache position `cache_pos`
 // q_proj: [Hq][2][D] (q_h then gate_h, full_attn_forward.rs:240-254).  inv_freq: the table
 // 1 / theta^(2i/rotary_dim), i < rotary_dim/2, computed on the host.
+// Token t of a chunk (blockIdx.y) has its inputs and outputs t rows further on, is rotated at
+// position pos + t and goes to cache position cache_pos + t.
 template <typename KV>
 __global__ void attn_prologue_kernel(int Hq, int Hkv, int D, int rotary_dim, float eps, int32_t pos,
                                      int64_t cache_pos, size_t plane_elems,
@@ -35,6 +37,16 @@ __global__ void attn_prologue_kernel(int Hq, int Hkv, int D, int rotary_dim, flo
     __shared__ float s_y[256];
     __shared__ float s_part[4];
     const int b = blockIdx.x, x = threadIdx.x;
+    {
+        const size_t t = blockIdx.y;
+        pos += (int32_t)t;
+        cache_pos += (int64_t)t;
+        q_proj += t * Hq * 2 * D;
+        k_in += t * Hkv * D;
+        v_in += t * Hkv * D;
+        q_out += t * Hq * D;
+        gate_out += t * Hq * D;
+    }
     if (b >= Hq + Hkv) {  // v is cached as it comes
         const int kvh = b - Hq - Hkv;
         v_tiled[(size_t)kvh * plane_elems + KvTile<KV>::v_off(cache_pos, x, D)] = to_kv<KV>(v_in[(size_t)kvh * D + x]);
@@ -68,7 +80,7 @@ __global__ void attn_prologue_kernel(int Hq, int Hkv, int D, int rotary_dim, flo
     else k_tiled[(size_t)h * plane_elems + KvTile<KV>::k_off(cache_pos, x, D)] = to_kv<KV>(r);
 }
 
-int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
+int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps, int n_tok,
                          int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,
                          const uint16_t *k_norm, const float *inv_freq, const float *q_proj, const float *k_in,
                          const float *v_in, float *q_out, float *gate_out, void *k_tiled, void *v_tiled) {
@@ -76,12 +88,14 @@ int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, in
     if (rotary_dim <= 0 || rotary_dim > D || (rotary_dim & 1))
         return fail(MFA_ERR_INVALID, "attention prologue: rotary_dim %d must be even and in (0, head_dim]", rotary_dim);
     if (pos < 0) return fail(MFA_ERR_INVALID, "attention prologue: pos %d < 0", pos);
+    if (n_tok <= 0 || n_tok > 65535) return fail(MFA_ERR_INVALID, "attention prologue: %d tokens (1..65535 per launch)", n_tok);
+    if ((int64_t)pos + n_tok - 1 > INT32_MAX) return fail(MFA_ERR_INVALID, "attention prologue: position overflow");
     if (kv_dtype == MFA_KV_BF16)
-        hipLaunchKernelGGL((attn_prologue_kernel<uint16_t>), dim3(Hq + 2 * Hkv), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
+        hipLaunchKernelGGL((attn_prologue_kernel<uint16_t>), dim3(Hq + 2 * Hkv, n_tok), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
                            eps, pos, cache_pos, plane_elems, q_norm, k_norm, inv_freq, q_proj, k_in, v_in, q_out,
                            gate_out, (uint16_t *)k_tiled, (uint16_t *)v_tiled);
     else
-        hipLaunchKernelGGL((attn_prologue_kernel<float>), dim3(Hq + 2 * Hkv), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
+        hipLaunchKernelGGL((attn_prologue_kernel<float>), dim3(Hq + 2 * Hkv, n_tok), dim3(D), 0, s, Hq, Hkv, D, rotary_dim,
                            eps, pos, cache_pos, plane_elems, q_norm, k_norm, inv_freq, q_proj, k_in, v_in, q_out,
                            gate_out, (float *)k_tiled, (float *)v_tiled);
     MFA_HIP(hipGetLastError());

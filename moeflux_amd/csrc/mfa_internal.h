@@ -142,6 +142,8 @@ struct Ctx {
     float *inv_freq = nullptr;
     int32_t rotary_dim = 0;
     float *qg_stage = nullptr;   // q and gate of mfa_full_attn_step, 2 * q_dim floats
+    float *qg_chunk = nullptr;   // the same for a chunk of tokens (mfa_prefill_full_attn), grown on demand
+    size_t qg_chunk_elems = 0;
     int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
     size_t plane_elems = 0;     // elements of one (layer, K|V, kv head) plane
     // split-K workspace
@@ -224,7 +226,7 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
 size_t matvec_tiled_words(int out_dim, int in_dim);
 int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, uint32_t *tiled);
 // attn_prologue.hip: q/gate split, per-head norms, rotation, cache append of one token.
-int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps,
+int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps, int n_tok,
                          int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,
                          const uint16_t *k_norm, const float *inv_freq, const float *q_proj, const float *k_in,
                          const float *v_in, float *q_out, float *gate_out, void *k_tiled, void *v_tiled);

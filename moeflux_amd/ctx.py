@@ -177,6 +177,18 @@ class Ctx:
         _chk(self.lib.mfa_full_attn_step(self.h, layer, pos, _p(qp), _p(k), _p(v), _p(out)), "mfa_full_attn_step")
         return out
 
+    def prefill_full_attn(self, layer, pos0, q_proj_out, k, v) -> np.ndarray:
+        """The layer step for a chunk of tokens at positions pos0, pos0 + 1, ...: [T, q_dim]."""
+        cfg = self.cfg
+        qp = _f32(q_proj_out)
+        T = qp.size // (2 * cfg.q_dim)
+        qp = _f32(qp, 2 * T * cfg.q_dim, "q_proj_out")
+        k, v = _f32(k, T * cfg.kv_dim, "k"), _f32(v, T * cfg.kv_dim, "v")
+        out = np.empty((T, cfg.q_dim), dtype=np.float32)
+        _chk(self.lib.mfa_prefill_full_attn(self.h, layer, pos0, T, _p(qp), _p(k), _p(v), _p(out)),
+             "mfa_prefill_full_attn")
+        return out
+
     def prefill_attn(self, layer, q, q_gate, k, v) -> np.ndarray:
         q = _f32(q)
         T = q.size // self.cfg.q_dim

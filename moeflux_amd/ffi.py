@@ -59,6 +59,8 @@ SIGNATURES = {
     "mfa_attn_prologue_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_full_attn_step_dev": (C.c_int, [vp, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
+    "mfa_prefill_full_attn": (C.c_int, [vp, C.c_int32, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
+    "mfa_prefill_full_attn_dev": (C.c_int, [vp, C.c_int32, C.c_int32, C.c_int32, f32p, f32p, f32p, f32p]),
     "mfa_dequant_matvec_4bit_dev": (C.c_int, [vp, C.c_int32, vp]),
     "mfa_dequant_matvec_4bit_tiled_dev": (C.c_int, [vp, C.c_int32, vp]),
     "mfa_matvec_tiled_words": (C.c_int64, [C.c_int32, C.c_int32]),

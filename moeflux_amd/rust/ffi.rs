@@ -69,6 +69,10 @@ extern "C" {
         k: *const f32, v: *const f32, q_out: *mut f32, q_gate_out: *mut f32) -> c_int;
     pub fn mfa_full_attn_step_dev(ctx: *mut mfa_ctx, layer: i32, pos: i32, q_proj_out: *const f32,
         k: *const f32, v: *const f32, out: *mut f32) -> c_int;
+    pub fn mfa_prefill_full_attn(ctx: *mut mfa_ctx, layer: i32, pos0: i32, t: i32, q_proj_out: *const f32,
+        k: *const f32, v: *const f32, out: *mut f32) -> c_int;
+    pub fn mfa_prefill_full_attn_dev(ctx: *mut mfa_ctx, layer: i32, pos0: i32, t: i32,
+        q_proj_out_dev: *const f32, k_dev: *const f32, v_dev: *const f32, out_dev: *mut f32) -> c_int;
     // projections either side of the core
     pub fn mfa_dequant_matvec_4bit_dev(ctx: *mut mfa_ctx, n: i32, specs: *const mfa_matvec_spec) -> c_int;
     pub fn mfa_dequant_matvec_4bit_tiled_dev(ctx: *mut mfa_ctx, n: i32, specs: *const mfa_matvec_spec) -> c_int;

@@ -83,6 +83,58 @@ def test_full_attn_steps_equal_the_reference_composition(mfa, oracle, bf16):
         assert c.kv_len(0) == n
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("Hq,Hkv,d,L0,T", [(32, 2, 256, 0, 70), (8, 2, 64, 5, 3), (32, 4, 128, 100, 513), (16, 4, 64, 37, 1)])
+def test_chunk_layer_step_equals_the_token_loop(mfa, oracle, bf16, Hq, Hkv, d, L0, T):
+    """A chunk of T tokens through norms, rotation, append and causal attention in one call, after
+    L0 tokens fed one by one: the same cache rows and, to the tolerance, the same outputs as the
+    loop of single-token steps that eval_prompt runs (riir/mod.rs:1196-1214); and the oracle's
+    composition for the chunk's last token."""
+    rng, qn, kn = _case(T + L0, Hq, Hkv, d)
+    n = L0 + T
+    qp = rng.standard_normal((n, Hq * 2 * d)).astype(np.float32)
+    k = rng.standard_normal((n, Hkv * d)).astype(np.float32)
+    v = rng.standard_normal((n, Hkv * d)).astype(np.float32)
+    with _ctx(mfa, Hq, Hkv, d, n + 1, bf16=bf16) as a, _ctx(mfa, Hq, Hkv, d, n + 1, bf16=bf16) as b:
+        for c in (a, b):
+            c.set_full_weights(0, qn, kn)
+            for t in range(L0):
+                c.full_attn_step(0, t, qp[t], k[t], v[t])
+        loop = np.stack([a.full_attn_step(0, L0 + t, qp[L0 + t], k[L0 + t], v[L0 + t]) for t in range(T)])
+        chunk = b.prefill_full_attn(0, L0, qp[L0:], k[L0:], v[L0:])
+        assert a.kv_len(0) == b.kv_len(0) == n
+        (ka, va), (kb, vb) = a.kv_export(0), b.kv_export(0)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+        assert chunk.shape == loop.shape and rel_err(chunk, loop) <= (1e-4 if bf16 else TOL_F32)
+        # a further single step continues from the chunk's cache as from the loop's
+        x = rng.standard_normal(Hq * 2 * d).astype(np.float32)
+        nk, nv = rng.standard_normal(Hkv * d).astype(np.float32), rng.standard_normal(Hkv * d).astype(np.float32)
+        assert np.array_equal(a.full_attn_step(0, n, x, nk, nv), b.full_attn_step(0, n, x, nk, nv))
+    rq, rg, _, _ = oracle.attn_prologue(n - 1, Hq, Hkv, d, d // 4, THETA, 1e-6, qn, kn, qp[-1], k[-1], v[-1])
+    ref = oracle.sdpa(n, Hq, Hkv, d, rq, rg, ka, va)
+    assert rel_err(chunk[-1], ref) <= (1e-4 if bf16 else TOL_F32)
+
+
+def test_chunk_layer_step_errors_append_nothing(mfa):
+    Hq, Hkv, d = 8, 2, 64
+    from moeflux_amd import MfaError, ffi
+    w = np.full(d, 0x3F80, np.uint16)
+    qp, kv = np.ones((4, Hq * 2 * d), np.float32), np.ones((4, Hkv * d), np.float32)
+    with _ctx(mfa, Hq, Hkv, d, 6) as c:
+        with pytest.raises(MfaError):
+            c.prefill_full_attn(0, 0, qp, kv, kv)         # weights not set
+        c.set_full_weights(0, w, w)
+        c.prefill_full_attn(0, 0, qp, kv, kv)
+        with pytest.raises(MfaError) as e:
+            c.prefill_full_attn(0, 4, qp, kv, kv)         # 4 + 4 > 6
+        assert e.value.code == ffi.ERR_OVERFLOW and c.kv_len(0) == 4
+        with pytest.raises(MfaError):
+            c.prefill_full_attn(0, -1, qp[:1], kv[:1], kv[:1])
+        assert c.kv_len(0) == 4
+        c.prefill_full_attn(0, 4, qp[:2], kv[:2], kv[:2])
+        assert c.kv_len(0) == 6
+
+
 def test_prologue_errors(mfa):
     Hq, Hkv, d = 8, 2, 64
     from moeflux_amd import MfaError
