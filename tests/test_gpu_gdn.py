@@ -221,3 +221,28 @@ def test_prompt_longer_than_one_segment(mfa):
     assert rel_err(out, ref_out) <= TOL_F32 and rel_err(ssm, ref_ssm) <= TOL_F32
     assert rel_err(out[4090:], ref_out[4090:]) <= 5e-5
     assert np.array_equal(conv.reshape(-1), ref_conv)
+
+
+def test_random_shapes_and_conv_widths(mfa):
+    """Seeded random head counts, both head widths, conv widths 2 to 8 and chunk lengths on either
+    side of the switch to the blocked form: a chunk after a few single steps, against the oracle's
+    sequential steps; outputs, the conv history (bit for bit) and the recurrent state."""
+    rng = np.random.default_rng(77)
+    shapes = [(128, 2, 4, 8, 5, 70), (64, 1, 2, 2, 0, 130), (128, 1, 1, 5, 9, 48), (64, 2, 8, 8, 17, 64)]
+    for _ in range(14):
+        Hk = int(rng.choice([1, 2, 4]))
+        K = int(rng.choice([2, 3, 4, 5, 8]))
+        shapes.append((int(rng.choice([64, 128])), Hk, Hk * int(rng.choice([1, 2, 4])), K, int(rng.integers(0, 2 * K)),
+                       int(rng.choice([1, 2, 7, 40, 48, 63, 64, 65, 130]))))
+    for case_no, (dk, Hk, Hv, K, pre, T) in enumerate(shapes):
+        case = GdnCase(500 + case_no, Hk, Hv, dk, dk, K=K, T=pre + T)
+        ref_out, ref_conv, ref_ssm = case.oracle()
+        with _ctx(mfa, case) as c:
+            c.linear_state_import(0, case.conv_state, case.ssm_state)
+            outs = [c.gdn_step(0, case.qkv[t], case.z[t], case.alpha[t], case.beta[t]) for t in range(pre)]
+            outs.extend(c.prefill_gdn(0, case.qkv[pre:], case.z[pre:], case.alpha[pre:], case.beta[pre:]))
+            conv, ssm = c.linear_state_export(0)
+        what = (case_no, Hk, Hv, dk, K, pre, T)
+        assert rel_err(np.stack(outs), ref_out) <= TOL_F32, what
+        assert np.array_equal(conv.reshape(-1), ref_conv), what
+        assert rel_err(ssm, ref_ssm) <= TOL_F32, what
