@@ -144,7 +144,7 @@ typedef struct mfa_matvec_spec {
  * attention core (shaders.metal:251-340; encoders gpu_matvec.rs; call sites
  * full_attn_forward.rs:193-227 for q/k/v_proj, linear_attn_forward.rs:560-605 for
  * in_proj_qkv/z/a/b, and o_proj / out_proj): n (1..8) products in one launch on
- * the context's stream.  in_dim a multiple of 64, at most 8192.  w and x must be
+ * the context's stream.  in_dim a multiple of 64, at most 16384.  w and x must be
  * 16-byte aligned (MFA_ERR_INVALID otherwise); scales and biases may start anywhere,
  * rows of them on 16-byte boundaries are read faster. */
 int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs);

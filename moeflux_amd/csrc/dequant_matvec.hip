@@ -322,7 +322,7 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
         if (!w[i] || !scales[i] || !biases[i] || !x[i] || !out[i]) return fail(MFA_ERR_INVALID, "dequant matvec: NULL pointer in product %d", i);
         if (out_dim[i] <= 0 || in_dim[i] <= 0) return fail(MFA_ERR_INVALID, "dequant matvec: non-positive shape in product %d", i);
         if (in_dim[i] % 64 != 0) return fail(MFA_ERR_INVALID, "dequant matvec: in_dim %d is not a multiple of the group size 64", in_dim[i]);
-        if (in_dim[i] > 8192) return fail(MFA_ERR_SHAPE, "dequant matvec: in_dim %d > 8192 not supported", in_dim[i]);
+        if (in_dim[i] > 16384) return fail(MFA_ERR_SHAPE, "dequant matvec: in_dim %d > 16384 not supported", in_dim[i]);
         sp.w[i] = w[i]; sp.scales[i] = scales[i]; sp.biases[i] = biases[i]; sp.x[i] = x[i]; sp.out[i] = out[i];
         sp.out_dim[i] = out_dim[i]; sp.in_dim[i] = in_dim[i];
         if ((uintptr_t)w[i] % 16 != 0 || (uintptr_t)x[i] % 16 != 0)
@@ -347,7 +347,8 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
     if (max_in <= 1024) MV_LAUNCH(1);
     else if (max_in <= 2048) MV_LAUNCH(2);
     else if (max_in <= 4096) MV_LAUNCH(4);
-    else MV_LAUNCH(8);
+    else if (max_in <= 8192) MV_LAUNCH(8);
+    else MV_LAUNCH(16);
 #undef MV_LAUNCH
     MFA_HIP(hipGetLastError());
     return MFA_OK;

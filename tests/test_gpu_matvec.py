@@ -29,11 +29,11 @@ def test_reference_unit_vectors(mfa):
 
 
 @pytest.mark.parametrize("out_dim,in_dim", [(1, 64), (5, 192), (33, 2048), (512, 4096), (100, 4160), (4096, 8192),
-                                            (16384, 4096), (37, 1024)])
+                                            (16384, 4096), (37, 1024), (7168, 16384), (100, 12288), (33, 8256)])
 def test_matvec_matches_oracle(mfa, oracle, out_dim, in_dim):
     """Projection shapes of the variants (q_proj 16384x4096, k/v_proj 512x4096, o_proj 4096x8192,
-    expert down_proj x1024) and ragged ones: row counts that do not fill a workgroup, widths that
-    do not fill the last 2048-input chunk."""
+    expert down_proj x1024, the latent-attention variants' o_proj 7168x16384) and ragged ones:
+    row counts that do not fill a workgroup, widths that do not fill the last 1024-input run."""
     rng = np.random.default_rng(out_dim + in_dim)
     packed, sc, bi = _weights(rng, out_dim, in_dim, oracle)
     x = rng.standard_normal(in_dim).astype(np.float32)
@@ -153,7 +153,7 @@ def test_tiled_weights_give_the_same_products(mfa, oracle):
     from moeflux_amd import Config, ffi
     from moeflux_amd.hip import DeviceArray
     rng = np.random.default_rng(10)
-    shapes = [(100, 4096), (33, 64), (512, 2048), (1, 1024), (17, 4160), (250, 3072), (16, 8192), (1000, 4096)]
+    shapes = [(100, 4096), (33, 64), (17, 9280), (1, 1024), (17, 4160), (250, 3072), (40, 16384), (1000, 4096)]
     keep, refs, outs, touts = [], [], [], []
     specs = (ffi.mfa_matvec_spec * len(shapes))()
     tspecs = (ffi.mfa_matvec_spec * len(shapes))()
@@ -211,3 +211,6 @@ def test_matvec_errors(mfa):
     assert lib.mfa_dequant_matvec_4bit(0, 64, 64, p(w), p(s), p(s), p(x), p(o)) == ffi.ERR_INVALID
     assert lib.mfa_dequant_matvec_4bit(1, 64, 64, None, p(s), p(s), p(x), p(o)) == ffi.ERR_INVALID
     assert lib.mfa_dequant_matvec_4bit(1, 64, 64, p(w), p(s), p(s), p(x), p(o)) == 0
+    # wider than the widest supported row (16384 inputs): refused, nothing is read
+    big_w, big_s, big_x = np.zeros(16448 // 8, np.uint32), np.zeros(16448 // 64, np.uint16), np.zeros(16448, np.float32)
+    assert lib.mfa_dequant_matvec_4bit(1, 16448, 64, p(big_w), p(big_s), p(big_s), p(big_x), p(o)) == ffi.ERR_SHAPE
