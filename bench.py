@@ -38,6 +38,36 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 C3_PARTIAL_TRAFFIC_BYTES = (65877 + 4128) * 1024
 
 
+def _bf16_bits(x):
+    """f32 -> bf16 bit patterns, round to nearest even (inputs here are finite)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+
+
+class _GdnInputs:
+    """Synthetic constants, state and T tokens of inputs of one Gated-DeltaNet layer at the step
+    shape the metric names: A_log = 0, dt_bias = 0, norm weight 1, conv weights ~ N(0, 0.5) in bf16."""
+
+    def __init__(self, seed, Hk, Hv, dk, dv, K=4, T=1, zero_state=False):
+        rng = np.random.default_rng(seed)
+        self.Hk, self.Hv, self.dk, self.dv, self.K, self.T = Hk, Hv, dk, dv, K, T
+        self.C = C = 2 * Hk * dk + Hv * dv
+        self.conv_w = _bf16_bits(rng.standard_normal(C * K) * 0.5)
+        self.a_log = np.zeros(Hv, np.float32)
+        self.dt_bias = _bf16_bits(np.zeros(Hv))
+        self.norm_w = _bf16_bits(np.ones(dv))
+        if zero_state:
+            self.conv_state = np.zeros((K - 1) * C, np.float32)
+            self.ssm_state = np.zeros(Hv * dv * dk, np.float32)
+        else:
+            self.conv_state = rng.standard_normal((K - 1) * C).astype(np.float32)
+            self.ssm_state = (rng.standard_normal(Hv * dv * dk) * 0.02).astype(np.float32)
+        self.qkv = rng.standard_normal((T, C)).astype(np.float32)
+        self.z = rng.standard_normal((T, Hv * dv)).astype(np.float32)
+        self.alpha = rng.standard_normal((T, Hv)).astype(np.float32)
+        self.beta = rng.standard_normal((T, Hv)).astype(np.float32)
+
+
 def _timed(ctx, lib, fn, steps, warmup):
     """Run fn(i) warmup+steps times; returns (wall ms per step, event ms per step)."""
     for i in range(warmup):
@@ -59,7 +89,6 @@ def _timed(ctx, lib, fn, steps, warmup):
 def bench_sdpa(name, Hq, Hkv, d, L, bf16, layers, steps, warmup, seed):
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
-    from oracle import cref
     lib = ffi.load()
     rng = np.random.default_rng(seed)
     kvd = Hkv * d
@@ -70,7 +99,7 @@ def bench_sdpa(name, Hq, Hkv, d, L, bf16, layers, steps, warmup, seed):
     base_k = rng.standard_normal((L + 8 * layers, kvd), dtype=np.float32)
     base_v = rng.standard_normal((L + 8 * layers, kvd), dtype=np.float32)
     if bf16:
-        base_k, base_v = cref.f32_to_bf16(base_k), cref.f32_to_bf16(base_v)
+        base_k, base_v = _bf16_bits(base_k), _bf16_bits(base_v)
     else:
         base_k *= qs
         base_v *= qs
@@ -115,9 +144,8 @@ def bench_sdpa(name, Hq, Hkv, d, L, bf16, layers, steps, warmup, seed):
 def bench_gdn(name, Hk, Hv, dk, dv, layers, steps, warmup, seed):
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
-    from tests.util import GdnCase
     lib = ffi.load()
-    case = GdnCase(seed, Hk, Hv, dk, dv, T=1, plain=True)
+    case = _GdnInputs(seed, Hk, Hv, dk, dv, T=1)
     ctx = Ctx(Config(num_layers=layers, full_attn_interval=layers + 1, linear_num_k_heads=Hk,
                      linear_num_v_heads=Hv, linear_key_dim=dk, linear_value_dim=dv))
     rng = np.random.default_rng(seed + 1)
@@ -158,7 +186,6 @@ def bench_prefill(steps, warmup, seed, T=512):
     chunk (configs[1] shape).  Every timed call uses a fresh layer, so kv_len0 = 0."""
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
-    from tests.util import GdnCase
     lib = ffi.load()
     Hq, Hkv, d = 32, 4, 128
     n = steps + warmup
@@ -214,7 +241,7 @@ def bench_prefill(steps, warmup, seed, T=512):
     for a in (dq, dg, dk, dv, do):
         a.free()
 
-    case = GdnCase(seed, 16, 32, 128, 128, T=T, zero_state=True, plain=True)
+    case = _GdnInputs(seed, 16, 32, 128, 128, T=T, zero_state=True)
     layers = 8
     ctx = Ctx(Config(num_layers=layers, full_attn_interval=layers + 1, linear_num_k_heads=16,
                      linear_num_v_heads=32))
@@ -247,17 +274,15 @@ def bench_sweep(steps, warmup, seed):
     on one stream (mfa_token_sweep_dev)."""
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
-    from oracle import cref
-    from tests.util import GdnCase
     lib = ffi.load()
     NL, Hq, Hkv, d, L = 48, 32, 2, 256, 8192
     cfg = Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                  kv_capacity=L, kv_dtype=ffi.KV_BF16, linear_num_k_heads=16, linear_num_v_heads=32)
     ctx = Ctx(cfg)
     rng = np.random.default_rng(seed)
-    case = GdnCase(seed, 16, 32, 128, 128, T=1, plain=True)
-    base_k = cref.f32_to_bf16(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
-    base_v = cref.f32_to_bf16(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
+    case = _GdnInputs(seed, 16, 32, 128, 128, T=1)
+    base_k = _bf16_bits(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
+    base_v = _bf16_bits(rng.standard_normal((L + 8 * 12, Hkv * d), dtype=np.float32))
     nf = nl = 0
     for i in range(NL):
         if cfg.is_full(i):
@@ -415,16 +440,15 @@ def bench_prologue(steps, warmup, seed):
     (prologue + split-K attention + merge over the grown cache, mfa_full_attn_step_dev)."""
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
-    from oracle import cref
     lib = ffi.load()
     Hq, Hkv, d, L = 32, 2, 256, 32768
     n = 2 * (steps + warmup) + 8
     ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                      kv_capacity=L + n, kv_dtype=ffi.KV_BF16))
     rng = np.random.default_rng(seed)
-    kv = cref.f32_to_bf16(rng.standard_normal((L, Hkv * d), dtype=np.float32))
+    kv = _bf16_bits(rng.standard_normal((L, Hkv * d), dtype=np.float32))
     ctx.kv_import(0, kv, kv)
-    w = cref.f32_to_bf16(np.ones(d, np.float32))
+    w = _bf16_bits(np.ones(d, np.float32))
     ctx.set_full_weights(0, w, w)
     qp = DeviceArray.from_host(rng.standard_normal(2 * Hq * d).astype(np.float32))
     k = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
@@ -460,13 +484,12 @@ def bench_snapshot(seed):
     memory (device reads and writes, conversion from and to the tiled cache, PCIe both ways);
     beside it the same state stored and restored as a device-resident checkpoint."""
     from moeflux_amd import Config, Ctx, ffi
-    from oracle import cref
     lib = ffi.load()
     NL, Hq, Hkv, d, L = 48, 32, 2, 256, 2048
     ctx = Ctx(Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                      kv_capacity=L, kv_dtype=ffi.KV_BF16, linear_num_k_heads=16, linear_num_v_heads=32))
     rng = np.random.default_rng(seed)
-    kv = cref.f32_to_bf16(rng.standard_normal((L, Hkv * d), dtype=np.float32))
+    kv = _bf16_bits(rng.standard_normal((L, Hkv * d), dtype=np.float32))
     for i in range(NL):
         if (i + 1) % 4 == 0:
             ctx.kv_import(i, kv, kv)
@@ -578,7 +601,6 @@ def cpu_baseline_all_cores(sample, Hq, Hkv, d, L):
 def cpu_secondary():
     """One-thread oracle timings of the secondary configurations, same shapes, bounded samples."""
     from oracle import cref
-    from tests.util import GdnCase
     rng = np.random.default_rng(1)
 
     def timed(fn, n):
@@ -595,7 +617,7 @@ def cpu_secondary():
     out = {}
     q, g, k, v = sdpa_inputs(32, 4, 128, 4096)
     out["c1_us_per_layer_token"] = timed(lambda: cref.sdpa(4096, 32, 4, 128, q, g, k, v), 5)
-    c = GdnCase(2, 16, 32, 128, 128, T=1, plain=True)
+    c = _GdnInputs(2, 16, 32, 128, 128, T=1)
     step = lambda: cref.gdn_step(16, 32, 128, 128, 4, 1e-6, c.conv_w, c.a_log, c.dt_bias, c.norm_w, c.qkv[0],
                                  c.z[0], c.alpha[0], c.beta[0], c.conv_state, c.ssm_state)
     out["c2_us_per_layer_token"] = timed(step, 20)
