@@ -68,22 +68,36 @@ class _GdnInputs:
         self.beta = rng.standard_normal((T, Hv)).astype(np.float32)
 
 
-def _timed(ctx, lib, fn, steps, warmup):
-    """Run fn(i) warmup+steps times; returns (wall ms per step, event ms per step)."""
+REPS = 11  # repetitions of the timed region; the median is reported
+
+
+def _timed(ctx, lib, fn, steps, warmup, reps=REPS):
+    """`warmup` untimed calls of fn(i), then `reps` repetitions of a timed region of exactly `steps`
+    calls, each bracketed by a stream synchronisation on both sides.  Returns the medians over the
+    repetitions of (wall ms per step, HIP-event ms per step); the events are recorded on the
+    library's stream just inside the wall-clock bracket."""
     for i in range(warmup):
         fn(i)
     lib.mfa_sync(ctx.h)
-    t0 = time.perf_counter()
-    lib.mfa_timer_start(ctx.h)
-    for i in range(steps):
-        fn(i)
+    walls, evs = [], []
     ms = C.c_float(0)
-    rc = lib.mfa_timer_stop(ctx.h, C.byref(ms))  # records the end event and waits for it
-    lib.mfa_sync(ctx.h)
-    wall = (time.perf_counter() - t0) * 1e3
-    if rc != 0:
-        raise RuntimeError("mfa_timer_stop failed")
-    return wall / steps, ms.value / steps
+    n = warmup
+    for _ in range(reps):
+        lib.mfa_sync(ctx.h)
+        t0 = time.perf_counter()
+        lib.mfa_timer_start(ctx.h)
+        for i in range(n, n + steps):
+            fn(i)
+        rc = lib.mfa_timer_stop(ctx.h, C.byref(ms))  # records the end event and waits for it: the stream is idle
+        wall = (time.perf_counter() - t0) * 1e3
+        if rc != 0:
+            raise RuntimeError("mfa_timer_stop failed")
+        walls.append(wall / steps)
+        evs.append(ms.value / steps)
+        n += steps
+    walls.sort()
+    evs.sort()
+    return walls[len(walls) // 2], evs[len(evs) // 2]
 
 
 def bench_sdpa(name, Hq, Hkv, d, L, bf16, layers, steps, warmup, seed):
@@ -188,7 +202,7 @@ def bench_prefill(steps, warmup, seed, T=512):
     from moeflux_amd.hip import DeviceArray
     lib = ffi.load()
     Hq, Hkv, d = 32, 4, 128
-    n = steps + warmup
+    n = REPS * steps + warmup
     rng = np.random.default_rng(seed)
     ctx = Ctx(Config(num_layers=n, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
                      head_dim=d, kv_capacity=T, kv_dtype=ffi.KV_BF16))
@@ -314,6 +328,7 @@ def bench_sweep(steps, warmup, seed):
     # one split-K launch + merge (all inputs of the token are known up front);
     # "per_layer": the 48 launch chains one after another, what a caller whose layers
     # depend on each other pays.
+    samples = {}
     for name, per_layer in (("per_kind", 0), ("per_layer", 1)):
         if lib.mfa_set_sweep_per_layer(ctx.h, per_layer) != 0:
             raise RuntimeError(ffi.last_error())
@@ -321,11 +336,24 @@ def bench_sweep(steps, warmup, seed):
         gbps = alg / (wall_ms * 1e-3) / 1e9
         res[name] = {"us_per_token_sweep": wall_ms * 1e3, "us_event": ev_ms * 1e3,
                      "us_per_layer_token": wall_ms * 1e3 / NL, "gbps": gbps,
-                     "pct_peak": 100.0 * gbps / HBM_PEAK_GBPS}
+                     "pct_peak": 100.0 * gbps / HBM_PEAK_GBPS,
+                     "pct_peak_event": 100.0 * alg / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        # one more sweep from a known state of the first DeltaNet layer, kept for the check against
+        # the CPU oracle (cpu_secondary): the first full-attention layer's and that layer's outputs
+        s0 = (rng.standard_normal(32 * 128 * 128) * 0.02).astype(np.float32)
+        for i in range(NL):   # every layer, so that all conv rings stand at the same slot again
+            if not cfg.is_full(i):
+                ctx.linear_state_import(i, case.conv_state, s0)
+        step(0)
+        ctx.sync()
+        samples[name] = {"full_out": fo.to_host()[0], "lin_out": lo.to_host()[0], "ssm0": s0}
+    sample = {"modes": samples, "q": fq.to_host()[0], "g": fg.to_host()[0], "k": base_k[:L], "v": base_v[:L],
+              "case": case, "x": lx.to_host()[0], "z": lz.to_host()[0], "a": la.to_host()[0], "b": lb.to_host()[0],
+              "shape": (Hq, Hkv, d, L)}
     ctx.close()
     for a in (fq, fg, fo, lx, lz, la, lb, lo):
         a.free()
-    return res
+    return res, sample
 
 
 def calibrate_copy(nbytes=64 << 20, reps=20):
@@ -342,6 +370,29 @@ def calibrate_copy(nbytes=64 << 20, reps=20):
     ctx.close()
     print(json.dumps({"copy_kernel": "plain_copy_kernel", "bytes_read_per_launch": nbytes,
                       "bytes_written_per_launch": nbytes, "launches": reps}))
+
+
+def calibrate_read(nbytes=64 << 20, reps=200):
+    """`--calibrate-read`: launches that only read 64 MiB (mfa_debug_read_dev), rotating over 8 buffers,
+    for several workgroup counts: what the memory system allows a launch of the headline kernel's size."""
+    from moeflux_amd import Config, Ctx, ffi
+    from moeflux_amd.hip import DeviceArray
+    lib = ffi.load()
+    ctx = Ctx(Config(num_layers=1, full_attn_interval=2, linear_num_k_heads=1, linear_num_v_heads=1))
+    bufs = [DeviceArray((nbytes,), np.uint8, zero=True) for _ in range(8)]
+    out = {"bytes_read_per_launch": nbytes, "launches_per_figure": reps, "by_workgroups": {}}
+    for wgs in (256, 512, 1024, 2048, 4096):
+        def step(i, wgs=wgs):
+            if lib.mfa_debug_read_dev(ctx.h, bufs[i % 8].ptr, nbytes, wgs) != 0:
+                raise RuntimeError(ffi.last_error())
+        _, ev_ms = _timed(ctx, lib, step, reps, 20, reps=5)
+        out["by_workgroups"][str(wgs)] = {"us_per_launch": ev_ms * 1e3, "gbps": nbytes / (ev_ms * 1e-3) / 1e9,
+                                          "pct_peak": 100.0 * nbytes / (ev_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    best = min(out["by_workgroups"].values(), key=lambda r: r["us_per_launch"])
+    out["best_us_per_launch"] = best["us_per_launch"]
+    out["best_pct_peak"] = best["pct_peak"]
+    ctx.close()
+    print(json.dumps(out))
 
 
 def cpu_baseline(sample, Hq, Hkv, d, L, budget_s=12.0):
@@ -442,7 +493,7 @@ def bench_prologue(steps, warmup, seed):
     from moeflux_amd.hip import DeviceArray
     lib = ffi.load()
     Hq, Hkv, d, L = 32, 2, 256, 32768
-    n = 2 * (steps + warmup) + 8
+    n = 2 * (REPS * steps + warmup) + 8
     ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                      kv_capacity=L + n, kv_dtype=ffi.KV_BF16))
     rng = np.random.default_rng(seed)
@@ -598,8 +649,10 @@ def cpu_baseline_all_cores(sample, Hq, Hkv, d, L):
             "sample": f"{n} calls, the {Hq} query heads of orc_sdpa spread over {cores} threads"}
 
 
-def cpu_secondary():
-    """One-thread oracle timings of the secondary configurations, same shapes, bounded samples."""
+def cpu_secondary(sweep_sample=None):
+    """One-thread oracle timings of the secondary configurations, same shapes, bounded samples;
+    with a sample of the 48-layer sweep (inputs and GPU outputs of its first full-attention and
+    first DeltaNet layer), the GPU outputs' error against the oracle on those inputs."""
     from oracle import cref
     rng = np.random.default_rng(1)
 
@@ -629,6 +682,18 @@ def cpu_secondary():
     q, g, k, v = sdpa_inputs(32, 2, 256, 8192)
     full = timed(lambda: cref.sdpa(8192, 32, 2, 256, q, g, k, v), 3)
     out["c5_us_per_token_sweep"] = 36 * out["c2_us_per_layer_token"] + 12 * full
+    if sweep_sample is not None:
+        sm = sweep_sample
+        Hq, Hkv, d, L = sm["shape"]
+        ref_f = cref.sdpa(L, Hq, Hkv, d, sm["q"], sm["g"], cref.bf16_to_f32(sm["k"]), cref.bf16_to_f32(sm["v"]))
+        cs = sm["case"]
+        chk = {}
+        for mode, o in sm["modes"].items():
+            ref_l, _, _ = cref.gdn_step(cs.Hk, cs.Hv, cs.dk, cs.dv, cs.K, 1e-6, cs.conv_w, cs.a_log, cs.dt_bias,
+                                        cs.norm_w, sm["x"], sm["z"], sm["a"], sm["b"], cs.conv_state, o["ssm0"])
+            chk[mode] = {"full_layer_rel_err": float(np.abs(o["full_out"] - ref_f).max() / np.abs(ref_f).max()),
+                         "deltanet_layer_rel_err": float(np.abs(o["lin_out"] - ref_l).max() / np.abs(ref_l).max())}
+        out["c5_gpu_vs_oracle"] = chk
     out["cores"] = 1
     out["kind"] = "port"
     out["sample"] = ("oracle functions at the full shapes: c1 5 calls, c2 20 calls, c4 attention one 512-token "
@@ -646,6 +711,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="launch only the plain copy kernel (for scaling memory counters) and exit")
+    ap.add_argument("--calibrate-read", action="store_true",
+                    help="time launches that only read 64 MiB (the memory system's ceiling at the headline launch size) and exit")
     ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
     ap.add_argument("--f4-len", type=int, default=0, help="one cache length for --only f4 (default: 4096 and 32768)")
     ap.add_argument("--only", choices=["c4", "c5", "f1", "f2", "f3", "f4"], default=None,
@@ -657,6 +724,9 @@ def main():
         sys.exit(2)
     if a.calibrate_copy:
         calibrate_copy()
+        return
+    if a.calibrate_read:
+        calibrate_read()
         return
 
     if a.only == "c4":
@@ -676,7 +746,10 @@ def main():
         print(json.dumps({"f4_mla_folded_sdpa": bench_mla(a.steps, a.warmup, 0xC0FFEE + 7, lens)}))
         return
     if a.only == "c5":
-        print(json.dumps({"c5_token_sweep_48_layers": bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)}))
+        r, sm = bench_sweep(a.steps, a.warmup, 0xC0FFEE + 5)
+        if not a.no_cpu:
+            r["gpu_vs_oracle"] = cpu_secondary(sm)["c5_gpu_vs_oracle"]
+        print(json.dumps({"c5_token_sweep_48_layers": r}))
         return
 
     Hq, Hkv, d, L = 32, 2, 256, 32768
@@ -685,6 +758,8 @@ def main():
         "metric": "attention us/layer/token + achieved HBM GB/s (% peak) at ctx 32K, 1 GPU",
         "value": head["us_per_layer_token"], "unit": "us/layer/token", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": head["us_per_layer_token"] / 1e3,
+        "us_event": head["us_event"], "timing": f"median of {REPS} repetitions of the {a.steps}-step region; value is wall clock "
+                                                 "with a stream synchronisation on both sides, us_event the same region between HIP events",
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 K/V, f32 accumulate",
         "data": "synthetic",
         "config": {"workload": "gated GQA decode, 32 Q / 2 KV heads, head_dim 256, kv_len 32768, "
@@ -710,13 +785,13 @@ def main():
         extra["c2_gated_deltanet_step"] = bench_gdn("c2", 16, 32, 128, 128, 160, a.steps, a.warmup,
                                                     0xC0FFEE + 2)
         extra["c4_prefill_chunk_512"] = bench_prefill(20, 5, 0xC0FFEE + 4)
-        extra["c5_token_sweep_48_layers"] = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
+        extra["c5_token_sweep_48_layers"], sweep_sample = bench_sweep(max(20, a.steps // 8), 5, 0xC0FFEE + 5)
         extra["f1_attention_prologue"] = bench_prologue(max(50, a.steps // 4), 10, 0xC0FFEE + 8)
         extra["f2_state_snapshot"] = bench_snapshot(0xC0FFEE + 9)
         extra["f3_projection_matvecs"] = bench_matvec(a.steps // 2, a.warmup, 0xC0FFEE + 6)
         extra["f4_mla_folded_sdpa"] = bench_mla(max(20, a.steps // 8), 5, 0xC0FFEE + 7)
         if not a.no_cpu:
-            extra["cpu_one_thread"] = cpu_secondary()
+            extra["cpu_one_thread"] = cpu_secondary(sweep_sample)
         line["extra"] = extra
     print(json.dumps(line))
 

@@ -435,6 +435,16 @@ int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t num_attn_heads, int32_t n
  * written, nbytes a multiple of 16): a launch of known memory traffic, used to scale
  * hardware memory counters when profiling.  No counterpart in the reference. */
 int mfa_debug_copy_dev(mfa_ctx *ctx, void *dst_dev, const void *src_dev, size_t nbytes);
+/* A launch on the context's stream that only reads nbytes (a multiple of 16) with the
+ * decode kernel's access pattern - `workgroups` workgroups of 256 threads, each reading
+ * one contiguous share with eight 1 KiB wave loads in flight, non-temporal - and computes
+ * nothing: the time the memory system allows a launch of that size, against which the
+ * decode kernel's own time is read.  No counterpart in the reference. */
+int mfa_debug_read_dev(mfa_ctx *ctx, const void *src_dev, size_t nbytes, int32_t workgroups);
+/* Fills the split-K workspace (partial outputs and their (max, sum) pairs) with a 32-bit
+ * pattern and waits.  Tests use it to show that no result depends on what the workspace
+ * held before a call (for instance NaN bit patterns).  No counterpart in the reference. */
+int mfa_debug_fill_workspace(mfa_ctx *ctx, uint32_t pattern);
 
 #pragma GCC visibility pop
 

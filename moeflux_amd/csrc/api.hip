@@ -294,6 +294,19 @@ static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
                                   sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok));
 }
 
+// What sdpa_dev could still refuse for n_tok tokens over a cache of kv_len positions, checked
+// (and the split-K workspace grown) while the cache is as the caller left it.
+static int sdpa_prepare(Ctx *c, int n_tok, int64_t kv_len) {
+    const mfa_config &g = c->cfg;
+    if (!c->forced_splits && !c->partial_only &&
+        sdpa_prefill_applies(g.kv_dtype, g.num_attn_heads, g.num_kv_heads, n_tok, kv_len, c->num_cus))
+        return MFA_OK;   // one launch, no workspace
+    const int64_t nhg = ((int64_t)n_tok * (g.num_attn_heads / g.num_kv_heads) + 15) / 16;
+    if (nhg > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
+    if (n_tok > 1) MFA_TRY(ensure_workspace(c, n_tok, kv_len));
+    return MFA_OK;
+}
+
 // n_tok tokens whose K/V rows are already in the cache (the last n_tok positions).
 static int sdpa_dev(Ctx *c, FullLayer *f, int n_tok, const float *q, const float *gate, float *out) {
     if (f->len <= 0) return fail(MFA_ERR_INVALID, "kv_len must be > 0 (got %d)", f->len);
@@ -541,6 +554,13 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
     return d2h_sync(c, out, c->stage + 2 * qd, qd * 4);
 }
 
+// Undo the appends of a call that failed after them, keeping the error of the failure.
+static void rollback_append(Ctx *c, FullLayer *f, int32_t len0) {
+    const std::string keep = g_last_error;
+    (void)truncate_full(c, *f, len0);
+    g_last_error = keep;
+}
+
 // n_tok tokens at positions pos .. pos + n_tok - 1, appended at the end of the layer's cache.
 static int prologue_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_proj, const float *k, const float *v,
                         float *q_out, float *gate_out, int32_t n_tok = 1) {
@@ -588,8 +608,11 @@ int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float
     MFA_TRY(full_layer(c, layer, &f));
     if (!q_proj_out_dev || !k_dev || !v_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
     const size_t qd = (size_t)c->q_dim();
+    const int32_t len0 = f->len;
     MFA_TRY(prologue_dev(c, f, pos, q_proj_out_dev, k_dev, v_dev, c->qg_stage, c->qg_stage + qd));
-    return sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, out_dev);
+    const int rc = sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, out_dev);
+    if (rc != MFA_OK) rollback_append(c, f, len0);
+    return rc;
 }
 
 int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out, const float *k,
@@ -604,8 +627,13 @@ int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_
     MFA_TRY(h2d(c, qp, q_proj_out, 2 * qd * 4));
     MFA_TRY(h2d(c, kk, k, kd * 4));
     MFA_TRY(h2d(c, vv, v, kd * 4));
+    const int32_t len0 = f->len;
     MFA_TRY(prologue_dev(c, f, pos, qp, kk, vv, c->qg_stage, c->qg_stage + qd));
-    MFA_TRY(sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, oo));
+    const int rc = sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, oo);
+    if (rc != MFA_OK) {
+        rollback_append(c, f, len0);
+        return rc;
+    }
     return d2h_sync(c, out, oo, qd * 4);
 }
 
@@ -631,15 +659,20 @@ int mfa_prefill_full_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t
         MFA_HIP(hipMalloc((void **)&c->qg_chunk, 2 * qd * sizeof(float)));
         c->qg_chunk_elems = 2 * qd;
     }
+    MFA_TRY(sdpa_prepare(c, T, (int64_t)f->len + T));
     // the whole chunk is normed, rotated and appended, then one causal pass: row t sees positions [0, len0 + t]
+    const int32_t len0 = f->len;
     const int kSeg = 32768;   // tokens per prologue launch (the grid's second dimension holds 65535)
-    for (int32_t off = 0; off < T; off += kSeg) {
+    int rc = MFA_OK;
+    for (int32_t off = 0; off < T && rc == MFA_OK; off += kSeg) {
         const int32_t n = T - off < kSeg ? T - off : kSeg;
-        MFA_TRY(prologue_dev(c, f, pos0 + off, q_proj_out_dev + (size_t)off * 2 * c->q_dim(),
-                             k_dev + (size_t)off * c->kv_dim(), v_dev + (size_t)off * c->kv_dim(),
-                             c->qg_chunk + (size_t)off * c->q_dim(), c->qg_chunk + qd + (size_t)off * c->q_dim(), n));
+        rc = prologue_dev(c, f, pos0 + off, q_proj_out_dev + (size_t)off * 2 * c->q_dim(),
+                          k_dev + (size_t)off * c->kv_dim(), v_dev + (size_t)off * c->kv_dim(),
+                          c->qg_chunk + (size_t)off * c->q_dim(), c->qg_chunk + qd + (size_t)off * c->q_dim(), n);
     }
-    return sdpa_dev(c, f, T, c->qg_chunk, c->qg_chunk + qd, out_dev);
+    if (rc == MFA_OK) rc = sdpa_dev(c, f, T, c->qg_chunk, c->qg_chunk + qd, out_dev);
+    if (rc != MFA_OK) rollback_append(c, f, len0);   // a launch refused after all: the cache is as before the call
+    return rc;
 }
 
 int mfa_prefill_full_attn(mfa_ctx *ctx, int32_t layer, int32_t pos0, int32_t T, const float *q_proj_out,
@@ -670,9 +703,13 @@ int mfa_prefill_attn_dev(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q_
     if ((int64_t)f->len + T > c->cfg.kv_capacity)
         return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + %d > capacity %d", f->len, T,
                     c->cfg.kv_capacity);
+    MFA_TRY(sdpa_prepare(c, T, (int64_t)f->len + T));
     // append the whole chunk, then one causal pass: row t sees positions [0, len0 + t]
-    MFA_TRY(kv_append_dev(c, f, k_dev, v_dev, T));
-    return sdpa_dev(c, f, T, q_dev, q_gate_dev, out_dev);
+    const int32_t len0 = f->len;
+    int rc = kv_append_dev(c, f, k_dev, v_dev, T);
+    if (rc == MFA_OK) rc = sdpa_dev(c, f, T, q_dev, q_gate_dev, out_dev);
+    if (rc != MFA_OK) rollback_append(c, f, len0);
+    return rc;
 }
 
 int mfa_prefill_attn(mfa_ctx *ctx, int32_t layer, int32_t T, const float *q, const float *q_gate,
@@ -1066,6 +1103,23 @@ int mfa_debug_copy_dev(mfa_ctx *ctx, void *dst_dev, const void *src_dev, size_t 
     Ctx *c = as_ctx(ctx);
     if (!c || !dst_dev || !src_dev) return fail(MFA_ERR_INVALID, "NULL argument");
     return launch_plain_copy(c->stream, dst_dev, src_dev, nbytes);
+}
+
+int mfa_debug_read_dev(mfa_ctx *ctx, const void *src_dev, size_t nbytes, int32_t workgroups) {
+    Ctx *c = as_ctx(ctx);
+    if (!c || !src_dev) return fail(MFA_ERR_INVALID, "NULL argument");
+    // the sink is 16 bytes per workgroup: the staging buffer holds them
+    MFA_TRY(ensure_stage(c, (size_t)(workgroups > 0 ? workgroups : 1) * 4));
+    return launch_plain_read(c->stream, src_dev, nbytes, workgroups, c->stage);
+}
+
+int mfa_debug_fill_workspace(mfa_ctx *ctx, uint32_t pattern) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (c->part_o) MFA_HIP(hipMemsetD32Async((hipDeviceptr_t)c->part_o, (int)pattern, c->part_o_elems, c->stream));
+    if (c->part_ml) MFA_HIP(hipMemsetD32Async((hipDeviceptr_t)c->part_ml, (int)pattern, c->part_ml_elems, c->stream));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    return MFA_OK;
 }
 
 /* ---- timing ------------------------------------------------------------------------ */

@@ -65,16 +65,52 @@ Sizes sizes_of(const Ctx *c) {
 // bytes of one plane's blocks that hold positions [0, len)
 size_t prefix_bytes(const Sizes &s, int32_t len) { return (size_t)((len + s.blk - 1) / s.blk) * s.block_bytes; }
 
-void release(Checkpoint &k) {
-    if (k.buf) (void)hipFree(k.buf);
+// An evicted or replaced checkpoint's buffer goes back to the pool for the next store: in
+// steady state (a rolling set of checkpoints) storing one allocates nothing.  The pool never
+// holds more buffers than checkpoints may be kept.
+void release(Ctx *c, Checkpoint &k) {
+    if (k.buf) {
+        if (c->checkpoint_pool.size() < c->max_checkpoints + 1) c->checkpoint_pool.emplace_back(k.buf, k.cap);
+        else (void)hipFree(k.buf);
+    }
     k.buf = nullptr;
+}
+
+// A buffer of at least `bytes`: the smallest pooled one that is large enough, else a new
+// allocation with a quarter of headroom (caches grow between stores), for which the largest
+// pooled buffer makes room.
+int acquire(Ctx *c, size_t bytes, Checkpoint &k) {
+    auto &pool = c->checkpoint_pool;
+    size_t best = pool.size();
+    for (size_t i = 0; i < pool.size(); i++)
+        if (pool[i].second >= bytes && (best == pool.size() || pool[i].second < pool[best].second)) best = i;
+    if (best != pool.size()) {
+        k.buf = pool[best].first;
+        k.cap = pool[best].second;
+        pool.erase(pool.begin() + best);
+        return MFA_OK;
+    }
+    if (!pool.empty()) {
+        size_t big = 0;
+        for (size_t i = 1; i < pool.size(); i++)
+            if (pool[i].second > pool[big].second) big = i;
+        (void)hipFree(pool[big].first);
+        pool.erase(pool.begin() + big);
+    }
+    const size_t cap = ((bytes + bytes / 4) | 255) + 1;
+    MFA_HIP(hipMalloc((void **)&k.buf, cap));
+    k.cap = cap;
+    return MFA_OK;
 }
 
 }  // namespace
 
 void drop_checkpoints(Ctx *c) {
-    for (auto &k : c->checkpoints) release(k);
+    for (auto &k : c->checkpoints)
+        if (k.buf) (void)hipFree(k.buf);
     c->checkpoints.clear();
+    for (auto &b : c->checkpoint_pool) (void)hipFree(b.first);
+    c->checkpoint_pool.clear();
 }
 
 }  // namespace mfa
@@ -96,7 +132,7 @@ int mfa_checkpoint_pos(mfa_ctx *ctx, int32_t pos) {
     }
     for (auto &l : c->lin) k.lin_step.push_back(l.step);
     k.bytes += s.ring_bytes + s.ssm_bytes;
-    MFA_HIP(hipMalloc((void **)&k.buf, k.bytes ? k.bytes : 16));
+    MFA_TRY(acquire(c, k.bytes, k));
     char *at = k.buf;
     int rc = MFA_OK;
     for (size_t i = 0; i < c->full.size() && rc == MFA_OK; i++) {
@@ -111,14 +147,14 @@ int mfa_checkpoint_pos(mfa_ctx *ctx, int32_t pos) {
     }
     if (rc == MFA_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail(MFA_ERR_HIP, "checkpoint copy failed");
     if (rc != MFA_OK) {
-        release(k);
+        release(c, k);
         return rc;
     }
     // a checkpoint already stored at this position is replaced and becomes the newest
     auto &cks = c->checkpoints;
     for (size_t i = 0; i < cks.size(); i++)
         if (cks[i].pos == pos) {
-            release(cks[i]);
+            release(c, cks[i]);
             cks.erase(cks.begin() + i);
             break;
         }
@@ -132,7 +168,7 @@ int mfa_checkpoint_pos(mfa_ctx *ctx, int32_t pos) {
                 break;
             }
         if (victim == cks.size()) break;
-        release(cks[victim]);
+        release(c, cks[victim]);
         cks.erase(cks.begin() + victim);
     }
     return MFA_OK;
@@ -149,6 +185,8 @@ int mfa_restore_to(mfa_ctx *ctx, int32_t pos) {
     const Checkpoint &k = cks[at_i];
     const Sizes s = sizes_of(c);
     const size_t Hkv = (size_t)c->cfg.num_kv_heads;
+    // Every copy is issued and waited for before a length or a ring position changes: a
+    // failure on the way leaves the context's bookkeeping where it was.
     const char *at = k.buf;
     for (size_t i = 0; i < c->full.size(); i++) {
         FullLayer &f = c->full[i];
@@ -161,18 +199,18 @@ int mfa_restore_to(mfa_ctx *ctx, int32_t pos) {
         MFA_TRY(copy_rows(c->stream, at, w, f.k, s.plane_bytes, w, Hkv));
         MFA_TRY(copy_rows(c->stream, at + Hkv * w, w, f.v, s.plane_bytes, w, Hkv));
         at += 2 * Hkv * w;
-        f.len = len;
     }
     if (!c->lin.empty()) {
         MFA_TRY(launch_plain_copy(c->stream, c->lin[0].conv_ring, at, s.ring_bytes));
         MFA_TRY(launch_plain_copy(c->stream, c->lin[0].ssm, at + s.ring_bytes, s.ssm_bytes));
-        for (size_t i = 0; i < c->lin.size(); i++) c->lin[i].step = k.lin_step[i];
     }
     MFA_HIP(hipStreamSynchronize(c->stream));
+    for (size_t i = 0; i < c->full.size(); i++) c->full[i].len = k.full_len[i];
+    for (size_t i = 0; i < c->lin.size(); i++) c->lin[i].step = k.lin_step[i];
     // later positions will be written afresh from here on: their checkpoints are void
     for (size_t i = cks.size(); i-- > 0;)
         if (cks[i].pos > pos) {
-            release(cks[i]);
+            release(c, cks[i]);
             cks.erase(cks.begin() + i);
         }
     return MFA_OK;

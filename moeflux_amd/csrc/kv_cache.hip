@@ -141,4 +141,39 @@ int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nby
     return MFA_OK;
 }
 
+// Streaming read of nbytes and nothing else (mfa_debug_read_dev): every workgroup reads one
+// contiguous share, eight 16-byte loads per lane in flight, each wave-level load 1 KiB
+// contiguous and non-temporal - the access pattern of the decode kernel without its arithmetic
+// or its partials.  Its time is what the memory system allows a launch of that size.
+__global__ __launch_bounds__(256) void plain_read_kernel(const uint4 *__restrict__ src, size_t n_per_block, size_t n,
+                                                         uint4 *__restrict__ sink) {
+    typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+    const size_t base = (size_t)blockIdx.x * n_per_block;
+    size_t end = base + n_per_block;
+    if (end > n) end = n;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (size_t i = base + threadIdx.x; i < end; i += 256 * 8) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const size_t j = i + (size_t)u * 256;
+            v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src) + (j < end ? j : i));
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc ^= v[u];
+    }
+    // never true for the buffers this is run on (the store keeps the loads alive)
+    if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u && acc.z == 0x0fedcba9u) sink[blockIdx.x] = __builtin_bit_cast(uint4, acc);
+}
+
+int launch_plain_read(hipStream_t stream, const void *src, size_t nbytes, int workgroups, void *sink) {
+    if (nbytes % 16 != 0 || nbytes == 0) return fail(MFA_ERR_INVALID, "read size must be a positive multiple of 16 bytes");
+    if (workgroups <= 0 || workgroups > 65536) return fail(MFA_ERR_INVALID, "1 to 65536 workgroups (got %d)", workgroups);
+    const size_t n = nbytes / 16;
+    const size_t per = (n + workgroups - 1) / workgroups;
+    hipLaunchKernelGGL(plain_read_kernel, dim3(workgroups), dim3(256), 0, stream, (const uint4 *)src, per, n, (uint4 *)sink);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
+}
+
 }  // namespace mfa

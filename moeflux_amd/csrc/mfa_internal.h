@@ -6,6 +6,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "moeflux_attn.h"
@@ -122,7 +123,8 @@ struct LinearLayer {
 struct Checkpoint {
     int32_t pos = 0;
     char *buf = nullptr;              // one allocation: K prefixes, V prefixes, rings, recurrent states
-    size_t bytes = 0;
+    size_t bytes = 0;                 // bytes in use
+    size_t cap = 0;                   // bytes allocated
     std::vector<int32_t> full_len;    // cache length of every full-attention layer
     std::vector<int64_t> lin_step;    // ring position of every linear layer
 };
@@ -164,6 +166,8 @@ struct Ctx {
     // checkpoints by position, least recently stored first (checkpoint.hip)
     std::vector<Checkpoint> checkpoints;
     size_t max_checkpoints = 4;       // DEFAULT_MAX_CHECKPOINTS, riir/mod.rs:105-109
+    // buffers of evicted or replaced checkpoints, kept for the next store (buffer, bytes allocated)
+    std::vector<std::pair<char *, size_t>> checkpoint_pool;
 
     int conv_dim() const {
         return 2 * cfg.linear_num_k_heads * cfg.linear_key_dim +
@@ -250,6 +254,8 @@ int launch_kv_zero(hipStream_t stream, int kv_dtype, int Hkv, int D, size_t plan
                    int64_t pos0, int64_t pos1, void *k_tiled, void *v_tiled);
 
 int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+// A launch that only reads nbytes (sink: 16 bytes per workgroup, never written in practice).
+int launch_plain_read(hipStream_t stream, const void *src, size_t nbytes, int workgroups, void *sink);
 
 // checkpoint.hip
 void drop_checkpoints(Ctx *c);   // frees every stored checkpoint (reset, destroy)

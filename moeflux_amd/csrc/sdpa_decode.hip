@@ -75,6 +75,8 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     if (b1 > nblk) b1 = nblk;
     const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
     if (b0 >= b1) {  // a split that lies wholly beyond what this group's rows may see
+        // Its rows of part_o stay unwritten: the merge gives a split whose maximum is -inf the
+        // weight 0 by selection, so whatever bytes the workspace holds there never enter a sum.
         if (wave == 0 && g == 0) {
             part_ml[pid * 32 + n] = neg_inf();
             part_ml[pid * 32 + 16 + n] = 0.f;
@@ -285,12 +287,16 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
 #pragma unroll
     for (int r = 0; r < kMergeRows; r++) {
         const float w = weight(mo[r]);
-        acc.x += w * rows[r].x; acc.y += w * rows[r].y; acc.z += w * rows[r].z; acc.w += w * rows[r].w;
+        if (w != 0.f) {   // a split no row of the group could see left its rows unwritten
+            acc.x += w * rows[r].x; acc.y += w * rows[r].y; acc.z += w * rows[r].z; acc.w += w * rows[r].w;
+        }
     }
     for (int s = sg + 16 * kMergeRows; s < nsplit; s += 16) {
         const float w = weight(ml[(size_t)s * 32]);
         const float4 v = *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0);
-        acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+        if (w != 0.f) {
+            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+        }
     }
     acc4[sg][dl] = acc;
     __syncthreads();
@@ -338,7 +344,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
 #pragma unroll
     for (int s = 0; s < NS; s++) {
         const float ws = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s));
-        acc += ws * rows[s];   // ws is 0 for s >= nsplit
+        if (ws != 0.f) acc += ws * rows[s];   // ws is 0 for s >= nsplit and for a split without rows (unwritten)
     }
     const float gt = gate ? 1.0f / (1.0f + expf(-gt_in)) : 1.0f;
     out[(size_t)bx * D + d] = (acc / den) * gt;

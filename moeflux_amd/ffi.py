@@ -105,6 +105,8 @@ SIGNATURES = {
     "mfa_debug_kv_offset": (C.c_int64, [i32, i32, C.c_int64, i32, i32]),
     "mfa_debug_num_splits": (i32, [i32, i32, i32, i32, C.c_int64, i32, i32]),
     "mfa_debug_copy_dev": (C.c_int, [vp, vp, vp, C.c_size_t]),
+    "mfa_debug_read_dev": (C.c_int, [vp, vp, C.c_size_t, C.c_int32]),
+    "mfa_debug_fill_workspace": (C.c_int, [vp, C.c_uint32]),
 }
 
 _lib = None

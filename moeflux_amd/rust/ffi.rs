@@ -148,4 +148,6 @@ extern "C" {
         kv_len: i64, num_cus: i32, forced_splits: i32) -> i32;
     pub fn mfa_debug_copy_dev(ctx: *mut mfa_ctx, dst_dev: *mut c_void, src_dev: *const c_void,
         nbytes: usize) -> c_int;
+    pub fn mfa_debug_read_dev(ctx: *mut mfa_ctx, src_dev: *const c_void, nbytes: usize, workgroups: i32) -> c_int;
+    pub fn mfa_debug_fill_workspace(ctx: *mut mfa_ctx, pattern: u32) -> c_int;
 }

@@ -6,7 +6,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from tests.util import TOL_F32, GdnCase, rel_err, sdpa_random_inputs
+from tests.util import TOL_F32, GdnCase, rel_err, rel_err_rows, sdpa_random_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -185,6 +185,88 @@ def test_token_sweep_equals_independent_calls(mfa, oracle, per_layer, ragged):
         assert rel_err(lo[j], ro) <= TOL_F32
         assert np.array_equal(new_states[j][0].reshape(-1), rc_)
         assert rel_err(new_states[j][1], rs) <= TOL_F32
+
+
+@pytest.mark.parametrize("forced", [0, 5])
+def test_stale_workspace_contents_never_reach_a_result(mfa, oracle, forced):
+    """A chunk whose first row group cannot see the cache's last split: 20 tokens of 32 Q / 2 KV
+    heads behind 1020 f32 positions are 65 blocks in 5 splits of 16, and token 0's rows end in
+    block 63, so their fifth split is empty and writes no partial rows.  The workspace is filled
+    with NaN bit patterns first: the merge must give such a split the weight 0 without touching
+    its rows.  Also with the split count forced."""
+    Hq, Hkv, d, T, L0 = 32, 2, 256, 20, 1020
+    rng = np.random.default_rng(1020)
+    k = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    v = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
+    q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
+    with _full_ctx(mfa, Hq, Hkv, d, L0 + T + 8) as c:
+        c.kv_import(0, k[:L0], v[:L0])
+        if forced:
+            c.set_num_splits(forced)
+        # a first call sizes the workspace for the chunk; the second runs over NaN
+        out0 = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+        c.memory_seq_rm(L0)
+        assert c.lib.mfa_debug_fill_workspace(c.h, 0x7FC00000) == 0
+        out = c.prefill_attn(0, q, g, k[L0:], v[L0:])
+    assert np.isfinite(out).all()
+    assert np.array_equal(out, out0)
+    assert rel_err(out, ref) <= TOL_F32
+    assert rel_err_rows(out, ref, d) <= 3e-5
+
+
+@pytest.mark.parametrize("per_layer", [0, 1])
+def test_config5_full_size_sweep(mfa, oracle, per_layer):
+    """The 48-layer hybrid stack at its own size: layers 3, 7, ..., 47 full attention
+    (variants.rs:258-264) with 32 Q / 2 KV heads, head_dim 256 and 8192 cached bf16 positions
+    each, the other 36 Gated-DeltaNet layers (16 / 32 heads, 128 x 128 states); distinct caches,
+    states, weights and inputs per layer.  One token's attention (the layer loop of
+    riir/mod.rs:1769-1888), launched once per layer kind and layer by layer: every layer's
+    output, conv history (bit for bit) and recurrent state against the oracle."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray
+    NL, Hq, Hkv, d, L = 48, 32, 2, 256, 8192
+    Hk, Hv, dk, dv, K = 16, 32, 128, 128, 4
+    cfg = Config(num_layers=NL, full_attn_interval=4, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=L, kv_dtype=1, linear_num_k_heads=Hk, linear_num_v_heads=Hv)
+    full_idx = [i for i in range(NL) if cfg.is_full(i)]
+    lin_idx = [i for i in range(NL) if not cfg.is_full(i)]
+    assert full_idx == list(range(3, NL, 4)) and len(lin_idx) == 36
+    rng = np.random.default_rng(0xC0FFEE + 5)
+    fulls = [sdpa_random_inputs(500 + i, Hq, Hkv, d, L, bf16=True) for i in full_idx]
+    cases = [GdnCase(600 + i, Hk, Hv, dk, dv) for i in lin_idx]
+    with mfa.Ctx(cfg) as c:
+        for i, (q, g, k, v) in zip(full_idx, fulls):
+            c.kv_import(i, k, v)
+        for i, cs in zip(lin_idx, cases):
+            c.set_linear_weights(i, cs.conv_w, cs.a_log, cs.dt_bias, cs.norm_w)
+            c.linear_state_import(i, cs.conv_state, cs.ssm_state)
+        dq = DeviceArray.from_host(np.array([f[0] for f in fulls]))
+        dg = DeviceArray.from_host(np.array([f[1] for f in fulls]))
+        dfo = DeviceArray((len(fulls), Hq * d), np.float32, zero=True)
+        dx = DeviceArray.from_host(np.array([cs.qkv[0] for cs in cases]))
+        dz = DeviceArray.from_host(np.array([cs.z[0] for cs in cases]))
+        da = DeviceArray.from_host(np.array([cs.alpha[0] for cs in cases]))
+        db = DeviceArray.from_host(np.array([cs.beta[0] for cs in cases]))
+        dlo = DeviceArray((len(cases), Hv * dv), np.float32, zero=True)
+        assert c.lib.mfa_set_sweep_per_layer(c.h, per_layer) == 0
+        assert c.lib.mfa_debug_fill_workspace(c.h, 0x7FC00000) == 0
+        rc = c.lib.mfa_token_sweep_dev(c.h, dq.ptr, dg.ptr, dfo.ptr, dx.ptr, dz.ptr, da.ptr, db.ptr, dlo.ptr)
+        assert rc == 0, ffi.last_error()
+        c.sync()
+        fo, lo = dfo.to_host(), dlo.to_host()
+        states = [c.linear_state_export(i) for i in lin_idx]
+    for j, (q, g, k, v) in enumerate(fulls):
+        ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+        assert rel_err(fo[j], ref) <= 1e-4, full_idx[j]
+        assert rel_err_rows(fo[j], ref, d) <= 1e-4, full_idx[j]
+    for j, cs in enumerate(cases):
+        ro, rconv, rssm = cs.oracle()
+        assert rel_err(lo[j], ro) <= TOL_F32, lin_idx[j]
+        assert rel_err_rows(lo[j], ro, dv) <= 3e-5, lin_idx[j]
+        assert np.array_equal(states[j][0].reshape(-1), rconv), lin_idx[j]
+        assert rel_err(states[j][1], rssm) <= TOL_F32, lin_idx[j]
 
 
 def test_state_operations_follow_the_reference(mfa, oracle):

@@ -17,6 +17,15 @@ def rel_err(a, b) -> float:
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
+def rel_err_rows(a, b, row_len) -> float:
+    """The same measure taken per row of `row_len` values (one head of one token), worst row:
+    max over rows of max|a_row - b_row| / max|b_row|.  A row of small values is held to its own
+    scale instead of hiding under a large neighbour."""
+    a = np.asarray(a, np.float64).reshape(-1, row_len)
+    b = np.asarray(b, np.float64).reshape(-1, row_len)
+    return float((np.abs(a - b).max(axis=1) / np.maximum(np.abs(b).max(axis=1), 1e-30)).max())
+
+
 def cosine(a, b) -> float:
     a = np.asarray(a, np.float64).reshape(-1)
     b = np.asarray(b, np.float64).reshape(-1)
