@@ -61,7 +61,24 @@ int ensure_stage(Ctx *c, size_t elems) {
 }
 
 static SdpaWorkspace workspace(Ctx *c) {
-    return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems};
+    return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems, &c->tickets, c->merge_wait,
+                         c->separate_merge};
+}
+
+// Ticket records for at least `groups` row groups (kv heads x 16-row groups of one launch), zeroed.
+static int ensure_tickets(Ctx *c, size_t groups) {
+    TicketRecords &t = c->tickets;
+    if (groups <= t.cap) return MFA_OK;
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    if (t.dev) MFA_HIP(hipFree(t.dev));
+    t = TicketRecords{};
+    size_t cap = 4096;
+    while (cap < groups) cap *= 2;
+    MFA_HIP(hipMalloc((void **)&t.dev, 2 * cap * sizeof(unsigned long long)));
+    MFA_HIP(hipMemsetAsync(t.dev, 0, 2 * cap * sizeof(unsigned long long), c->stream));
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    t.cap = cap;
+    return MFA_OK;
 }
 
 static int h2d(Ctx *c, void *dst, const void *src, size_t bytes) {
@@ -83,6 +100,7 @@ static void destroy(Ctx *c) {
         if (p) (void)hipFree(p);
     if (c->part_o) (void)hipFree(c->part_o);
     if (c->part_ml) (void)hipFree(c->part_ml);
+    if (c->tickets.dev) (void)hipFree(c->tickets.dev);
     if (c->stage) (void)hipFree(c->stage);
     if (c->gdn_scratch) (void)hipFree(c->gdn_scratch);
     if (c->qg_chunk) (void)hipFree(c->qg_chunk);
@@ -213,6 +231,7 @@ static int create(const mfa_config *cfg, Ctx **out) {
         c->part_ml_elems = sdpa_workspace_ml_elems(cfg->num_attn_heads, cfg->num_kv_heads, splits);
         MFA_HIP(hipMalloc((void **)&c->part_o, c->part_o_elems * sizeof(float)));
         MFA_HIP(hipMalloc((void **)&c->part_ml, c->part_ml_elems * sizeof(float)));
+        MFA_TRY(ensure_tickets(c, 4096));
     }
     if (nlin) {
         const size_t C = (size_t)c->conv_dim(), K = (size_t)cfg->conv_kernel_size;
@@ -290,6 +309,7 @@ static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
     const int Hq = g.num_attn_heads * layers, Hkv = g.num_kv_heads * layers;
     int splits = sdpa_pick_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
     if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
+    MFA_TRY(ensure_tickets(c, (size_t)Hkv * (((size_t)n_tok * (g.num_attn_heads / g.num_kv_heads) + 15) / 16)));
     return ensure_workspace_elems(c, sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok),
                                   sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok));
 }
@@ -471,6 +491,16 @@ int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits) {
     c->forced_splits = num_splits;
     // a forced count is used as given, so the workspace must hold it at any cache length
     if (num_splits > 0 && !c->full.empty()) MFA_TRY(ensure_workspace(c, 1, c->cfg.kv_capacity));
+    return MFA_OK;
+}
+
+int mfa_set_merge(mfa_ctx *ctx, int32_t in_launch, int32_t helper_polls) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (helper_polls < -1 || helper_polls > (1 << 20))
+        return fail(MFA_ERR_INVALID, "helper_polls must be -1 (default) or in [0, 2^20] (got %d)", helper_polls);
+    c->separate_merge = in_launch ? 0 : 1;
+    c->merge_wait = helper_polls < 0 ? kDefaultMergeWait : helper_polls;
     return MFA_OK;
 }
 

@@ -94,6 +94,20 @@ template <> struct KvTile<float> {
     }
 };
 
+// Ticket records of the merge that runs inside the split-K launch: two sets of `cap` 64-bit
+// words; launches alternate between the sets and each clears what the other set's last user
+// touched (sdpa_decode.hip).  Host-side bookkeeping of one stream's launches.
+struct TicketRecords {
+    unsigned long long *dev = nullptr;
+    size_t cap = 0;            // records per set
+    int cur = 0;               // set the next launch uses
+    size_t used[2] = {0, 0};   // records of each set that may be non-zero
+};
+
+// Polls a helper workgroup of the in-launch merge makes before it gives up (about 0.1 us of
+// sleep plus one read of the record each).
+static constexpr int kDefaultMergeWait = 24;
+
 // ---- context ----------------------------------------------------------------
 struct LinearWeights {
     uint16_t *conv_w = nullptr;  // [C, K] bf16
@@ -154,6 +168,9 @@ struct Ctx {
     size_t part_o_elems = 0, part_ml_elems = 0;
     int32_t forced_splits = 0;
     int32_t partial_only = 0;
+    TicketRecords tickets;      // of the merge inside the split-K launch
+    int32_t merge_wait = kDefaultMergeWait;
+    int32_t separate_merge = 1;   // the merge is a launch of its own unless mfa_set_merge asks otherwise
     // scratch of the Gated-DeltaNet chunk kernels (grown on demand)
     float *gdn_scratch = nullptr;
     size_t gdn_scratch_elems = 0;
@@ -192,6 +209,9 @@ struct SdpaWorkspace {
     float *part_o;
     float *part_ml;
     size_t part_o_elems, part_ml_elems;
+    TicketRecords *tickets = nullptr;   // null: the merge is always a second launch
+    int merge_wait = 0;                 // polls of a helper workgroup before it gives up
+    int separate_merge = 1;             // 0: merge inside the split-K launch (needs tickets)
 };
 bool sdpa_shape_supported(int kv_dtype, int head_dim);
 // Number of splits the launcher will use (for workspace sizing pass kv_len = capacity).

@@ -29,10 +29,14 @@
 //     v_mfma_f32_16x16x4_f32.  The query is pre-multiplied by scale*log2 e so a
 //     probability is one v_exp_f32.  One (max, sum, O[16, D]) partial per
 //     workgroup is written.
-//   sdpa_merge_kernel    log-sum-exp merge of the partials, normalisation and
-//     the sigmoid gate.
-#include "gdn_device.h"
-#include "sdpa_wave.h"
+//   The log-sum-exp merge of the partials, the normalisation and the sigmoid gate
+//   run in the same launch: every workgroup takes a ticket of its row group when its
+//   partial is visible device-wide, and the one that draws the last ticket (helped,
+//   when the group has many splits, by workgroups that arrived a moment earlier and
+//   looked on for a bounded time) combines the group's partials.  No workgroup ever
+//   depends on another one making progress.  sdpa_merge_kernel / sdpa_merge_few_kernel
+//   are the same merge as a launch of its own (the latent-cache attention uses them).
+#include "sdpa_merge.h"
 
 namespace mfa {
 
@@ -40,11 +44,40 @@ static constexpr int kMaxSplits = 1024;
 
 // part_o:  [kv head][head group][split][16 heads][D]
 // part_ml: [kv head][head group][split][2][16]   (max in log2 units, then sum)
+// The merge inside the split-K launch.  A row group's record is one 64-bit word, zero when the
+// launch starts: arrivals in the high half, claimed chunks of the group's output in the low half.
+//   * A workgroup makes its partial visible device-wide (release fence), then adds 1 to the
+//     arrivals with one device-scope atomic; the value that comes back is its ticket.  The one
+//     that draws the last ticket knows every partial of the group is complete.
+//   * Few splits (<= 16): that workgroup merges the whole group, all requests in flight at once.
+//   * Many splits: the group's output is cut into chunks and the workgroups of the first splits
+//     are helpers: a helper claims chunk `split` in the same atomic that takes its ticket, then
+//     reads the record a bounded number of times; when it sees the last arrival it merges its
+//     chunk.  A helper that gives up hands the chunk back (one atomic; should the last arrival
+//     have come in between, it merges the chunk after all).  The last arrival merges every chunk
+//     nobody held when it arrived.  Each chunk has exactly one owner, who only starts once all
+//     partials are visible, and no workgroup waits without a bound: progress never depends on
+//     which workgroups are resident.
+//   * Records are never reset by the launch that uses them: launches alternate between two sets
+//     of records, and each launch zeroes the records the previous user of the other set touched.
+struct FusedMerge {
+    unsigned long long *rec;    // this launch's records [kv head][row group]; null: no merge in this launch
+    unsigned long long *zero;   // records of the other set to clear, [0, n_zero)
+    int n_zero;
+    int wait;                   // polls a helper makes before it gives up
+    const float *gate;
+    float *out;
+};
+
+static constexpr int kFewSplits = 16;        // at most this many: merged by one workgroup in one go
+static constexpr int kMaxMergeChunks = 32;   // claim bits of a record
+
 template <typename KV, int D, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
     const float *__restrict__ q, int hpk, int Hq, int n_tok, int64_t kv_len0,
-    int blocks_per_split, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml) {
+    int blocks_per_split, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml,
+    FusedMerge fm) {
     using W = Wave<KV, D>;
     constexpr int NACC = W::NACC;
     constexpr int TPW = NACC / WAVES;  // output tiles owned by one wave
@@ -74,15 +107,20 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     int64_t b1 = b0 + blocks_per_split;
     if (b1 > nblk) b1 = nblk;
     const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
+    if (fm.rec && fm.n_zero > 0 && threadIdx.x == 0) {   // clear the other set's used records
+        const int nwg = gridDim.x * gridDim.y * gridDim.z;
+        for (int i = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; i < fm.n_zero; i += nwg)
+            fm.zero[i] = 0ull;
+    }
     if (b0 >= b1) {  // a split that lies wholly beyond what this group's rows may see
         // Its rows of part_o stay unwritten: the merge gives a split whose maximum is -inf the
         // weight 0 by selection, so whatever bytes the workspace holds there never enter a sum.
         if (wave == 0 && g == 0) {
-            part_ml[pid * 32 + n] = neg_inf();
-            part_ml[pid * 32 + 16 + n] = 0.f;
+            const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, neg_inf()), mlb, n * 4, 0, kThrough);
+            __builtin_amdgcn_raw_buffer_store_b32(0u, mlb, (16 + n) * 4, 0, kThrough);
         }
-        return;
-    }
+    } else {
 
     // ---- requests, in the order they are needed (loads return in order) ---------
     // Every load below is unconditional (indices are clamped instead), so that the
@@ -218,104 +256,129 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     l_run += lane_xor(l_run, 16);
     l_run += lane_xor(l_run, 32);
     if (g == 0) sl[wave][n] = l_run;
-    float *row = part_o + (pid * 16 + n) * D;
+    // stores that go through to memory: the partial is read by whichever workgroup merges the group
+    const __amdgpu_buffer_rsrc_t ob = buffer_of(part_o + pid * 16 * D);
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
         // tile dt, lane group g, element i is channel 16 dt + 4g + i of head n
-        const float4 v = {o[t][0], o[t][1], o[t][2], o[t][3]};
-        *(float4 *)(row + 16 * (wave * TPW + t) + 4 * g) = v;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o[t]), ob,
+                                               (n * D + 16 * (wave * TPW + t) + 4 * g) * 4, 0, kThrough);
     }
     __syncthreads();
     if (wave == 0 && g == 0) {
         float lsum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) lsum += sl[w][n];
-        part_ml[pid * 32 + n] = m_run;
-        part_ml[pid * 32 + 16 + n] = lsum;
+        const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, m_run), mlb, n * 4, 0, kThrough);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, lsum), mlb, (16 + n) * 4, 0, kThrough);
+    }
+    }  // a split with positions
+
+    if (!fm.rec) return;   // partials only (uniform over the launch)
+
+    // ---- ticket, and the merge by whoever it falls to -----------------------------------------
+    constexpr int TEAMS = WAVES / 4;                 // 256-thread teams of the many-split merge
+    constexpr int PER_ROW = D / 64;                  // 64-output units per row
+    constexpr int UNITS = 16 * PER_ROW;              // units of a row group
+    __shared__ float4 acc4[TEAMS][2][16][16];
+    __shared__ unsigned int s_own;                   // chunks this workgroup merges (bit set), 0: none
+    const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
+    const MergeOut mo{fm.gate, fm.out, hpk, Hq, n_tok, D};
+    const bool few = nsplit <= kFewSplits;
+    // chunks of the many-split merge: a power of two, at most one per split, at most 32, and
+    // not finer than what the workgroup's teams merge in one pass
+    int nchunks = UNITS / TEAMS < kMaxMergeChunks ? UNITS / TEAMS : kMaxMergeChunks;
+    while (nchunks > nsplit) nchunks >>= 1;
+    const bool helper = !few && split < nchunks;
+
+    // The partial was written with stores that go through to memory: once every wave has counted
+    // its own off it is visible device-wide, and the ticket is taken after that.
+    wait_for_stores();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long *rec = fm.rec + (size_t)kvh * nhg + hg;
+        const unsigned long long one = 1ull << 32, bit = helper ? (1ull << split) : 0ull;
+        const unsigned long long old = __hip_atomic_fetch_add(rec, one + bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned int own = 0;
+        if ((int)(old >> 32) == nsplit - 1) {
+            // the last arrival: every chunk no helper held at this moment (its own included)
+            const unsigned int all = few ? 1u : (nchunks == 32 ? 0xffffffffu : (1u << nchunks) - 1u);
+            own = all & ~(unsigned int)old;
+        } else if (helper) {
+            bool complete = false;
+            for (int i = 0; i < fm.wait && !complete; i++) {
+                __builtin_amdgcn_s_sleep(2);
+                complete = (int)(__hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == nsplit;
+            }
+            if (!complete) {
+                // give the chunk back; if the last arrival has been in the meantime, it left the chunk to us
+                const unsigned long long was = __hip_atomic_fetch_add(rec, 0ull - bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                complete = (int)(was >> 32) == nsplit;
+            }
+            if (complete) own = (unsigned int)bit;
+        }
+        s_own = own;
+    }
+    __syncthreads();
+    unsigned int own = s_own;
+    if (own == 0) return;
+    // every split's partial is in memory from here on; the reader's loads go there for it
+    const PartialsThrough rd(part_o, part_ml, pid0, D);
+
+    if (few) {
+        // the whole group in passes of WAVES * UPW units, every request of a pass in flight at once
+        if (nsplit <= 8) {
+            constexpr int UPW = 8;
+            for (int u0 = 0; u0 < UNITS; u0 += WAVES * UPW)
+                merge_few_units<8, UPW>(rd, nsplit, kvh, hg, u0 + wave * UPW, UNITS, mo, lane);
+        } else {
+            constexpr int UPW = 4;
+            for (int u0 = 0; u0 < UNITS; u0 += WAVES * UPW)
+                merge_few_units<16, UPW>(rd, nsplit, kvh, hg, u0 + wave * UPW, UNITS, mo, lane);
+        }
+        return;
+    }
+    const int team = threadIdx.x >> 8, ttid = threadIdx.x & 255;
+    const int upc = UNITS / nchunks;                 // units of a chunk, consecutive: a power of two
+    while (own) {
+        const int c = __builtin_ctz(own);
+        own &= own - 1;
+        // a chunk's units lie in one row when upc <= PER_ROW, else it is whole rows; a team
+        // takes spans of up to two units (128 channels) of one row at a time
+        constexpr int SPAN = PER_ROW >= 2 ? 2 : 1;   // units per team pass, at most
+        const int span = upc / TEAMS < SPAN ? 1 : SPAN;
+        for (int u0 = c * upc; u0 < (c + 1) * upc; u0 += TEAMS * span) {
+            const int u = u0 + team * span;
+            const bool in = u < (c + 1) * upc;
+            const int nn = (in ? u : 0) / PER_ROW, c0 = ((in ? u : 0) % PER_ROW) * 64;
+            const int64_t orow = mo.row(kvh, hg * 16 + nn);
+            const bool active = in && orow >= 0;
+            if (span == 2)
+                merge_span<2>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team]);
+            else
+                merge_span<1>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team]);
+        }
     }
 }
 
-// grid (Hq, D/64), 256 threads: 16 lanes x float4 cover 64 outputs of one split's row,
-// 16 such rows per pass.  Every wave forms the overall maximum and the denominator by
-// itself (each lane reads the (max, sum) of splits lane, lane + 64, ..., and the maxima of
-// the splits whose rows it combines), so nothing waits for another wave until the 16 row
-// sums meet in LDS, and every request - split statistics, rows, gate - is made before the
-// first value is used: one memory round trip and one barrier.
-static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
+
+// The same merge as a launch of its own.
+// grid (n_tok * Hq, D/64), 256 threads: one 64-output unit per workgroup.
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
-    __shared__ float4 acc4[16][16];
+    __shared__ float4 acc4[1][16][16];
     // blockIdx.x = token * Hq + head; its row in the kv head's row list is token*hpk + head%hpk
     const int h = blockIdx.x % Hq, tok = blockIdx.x / Hq;
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int dl = tid & 15, sg = tid >> 4;  // 16 float4 lanes x 16 split lanes
-    const int d0 = blockIdx.y * 64 + dl * 4;
-    const float *ml = part_ml + pid0 * 32 + n;   // split s: maximum at ml[32 s], sum at ml[32 s + 16]
-
-    float ms[4], ls[4];   // splits lane + 64 r (the first 256; beyond that, see the loops below)
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int s = lane + 64 * r;
-        ms[r] = (s < nsplit) ? ml[(size_t)s * 32] : neg_inf();
-        ls[r] = (s < nsplit) ? ml[(size_t)s * 32 + 16] : 0.f;
-    }
-    float mo[kMergeRows];   // maxima of the splits whose rows this thread combines
-    float4 rows[kMergeRows];
-#pragma unroll
-    for (int r = 0; r < kMergeRows; r++) {
-        const int s = sg + 16 * r;
-        mo[r] = (s < nsplit) ? ml[(size_t)s * 32] : neg_inf();
-        rows[r] = (s < nsplit) ? *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0)
-                               : float4{0.f, 0.f, 0.f, 0.f};
-    }
-    const float gt_in = (gate && tid < 64) ? gate[(size_t)blockIdx.x * D + blockIdx.y * 64 + tid] : 0.f;
-
-    float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
-    for (int s = lane + 256; s < nsplit; s += 64) m = fmaxf(m, ml[(size_t)s * 32]);
-    const float M = wave_max(m);
-    auto weight = [&](float ms_) { return (ms_ == neg_inf()) ? 0.f : fast_exp2(ms_ - M); };
-    float den = 0.f;
-#pragma unroll
-    for (int r = 0; r < 4; r++) den += weight(ms[r]) * ls[r];
-    for (int s = lane + 256; s < nsplit; s += 64) den += weight(ml[(size_t)s * 32]) * ml[(size_t)s * 32 + 16];
-    den = group_sum<64>(den);
-
-    float4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < kMergeRows; r++) {
-        const float w = weight(mo[r]);
-        if (w != 0.f) {   // a split no row of the group could see left its rows unwritten
-            acc.x += w * rows[r].x; acc.y += w * rows[r].y; acc.z += w * rows[r].z; acc.w += w * rows[r].w;
-        }
-    }
-    for (int s = sg + 16 * kMergeRows; s < nsplit; s += 16) {
-        const float w = weight(ml[(size_t)s * 32]);
-        const float4 v = *(const float4 *)(part_o + ((pid0 + s) * 16 + n) * D + d0);
-        if (w != 0.f) {
-            acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
-        }
-    }
-    acc4[sg][dl] = acc;
-    __syncthreads();
-    if (tid < 64) {
-        // thread -> one scalar output: float4 lane tid/4, component tid%4
-        const int ql = tid >> 2, qc = tid & 3;
-        float t = 0.f;
-#pragma unroll
-        for (int x = 0; x < 16; x++) t += ((const float *)&acc4[x][ql])[qc];
-        const int d = blockIdx.y * 64 + tid;
-        const float gt = gate ? 1.0f / (1.0f + expf(-gt_in)) : 1.0f;
-        out[(size_t)blockIdx.x * D + d] = (t / den) * gt;
-    }
+    merge_span<1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate, out,
+                  threadIdx.x, acc4);
 }
 
-// The merge for few splits (at most NS = 8 or 16, what a launch over many layers or row groups
-// ends up with): one wave per 64 outputs of a (token, head) row, four such units per workgroup,
-// no LDS and no barrier (the 12-layer sweep's merge: 5.0 -> 3 us; no gain from 32 splits on).  Lane s holds split s's (max, sum); a
-// lane's output is the weighted sum of one float per split, all requested before the first use.
+// Few splits (at most NS = 8 or 16, what a launch over many layers or row groups ends up
+// with): one wave per 64 outputs of a (token, head) row, four such units per workgroup.
 template <int NS>
 __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
@@ -327,27 +390,9 @@ __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const int h = bx % Hq, tok = bx / Hq;
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const float *ml = part_ml + pid0 * 32 + n;
-    const int d = by * 64 + lane;
-    const int sl = lane < nsplit ? lane : nsplit - 1;
-    const float m_in = ml[(size_t)sl * 32], l_in = ml[(size_t)sl * 32 + 16];
-    float rows[NS];
-#pragma unroll
-    for (int s = 0; s < NS; s++) rows[s] = part_o[((pid0 + (s < nsplit ? s : nsplit - 1)) * 16 + n) * D + d];
-    const float gt_in = gate ? gate[(size_t)bx * D + d] : 0.f;
-
-    const float ms = lane < nsplit ? m_in : neg_inf();
-    const float M = wave_max(ms);
-    const float w = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
-    const float den = group_sum<64>(w * (lane < nsplit ? l_in : 0.f));
-    float acc = 0.f;
-#pragma unroll
-    for (int s = 0; s < NS; s++) {
-        const float ws = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s));
-        if (ws != 0.f) acc += ws * rows[s];   // ws is 0 for s >= nsplit and for a split without rows (unwritten)
-    }
-    const float gt = gate ? 1.0f / (1.0f + expf(-gt_in)) : 1.0f;
-    out[(size_t)bx * D + d] = (acc / den) * gt;
+    const int u = n * per_row + by;   // the unit's index inside its row group
+    const MergeOut mo{gate, out, hpk, Hq, (int)(((int64_t)n_units / per_row) / Hq), D};
+    merge_few_units<NS, 1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, kvh, hg, u, u + 1, mo, lane);
 }
 
 static void launch_merge_kernels(hipStream_t stream, const float *part_o, const float *part_ml, int splits, int hpk,
@@ -432,25 +477,25 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok) {
 template <typename KV, int D, int WAVES>
 static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
                            size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                           int64_t kv_len0, int bps, float qscale, float *po, float *pml) {
+                           int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm) {
     hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES>), grid, dim3(WAVES * 64), 0, stream,
                        (const KV *)k, (const KV *)v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                       qscale, po, pml);
+                       qscale, po, pml, fm);
 }
 
 template <typename KV, int D>
 static void launch_partial_w(int waves, hipStream_t stream, dim3 grid, const void *k, const void *v,
                              size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                             int64_t kv_len0, int bps, float qscale, float *po, float *pml) {
+                             int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm) {
     if constexpr (D >= 128) {
         if (waves == 8) {
             launch_partial<KV, D, 8>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                                     qscale, po, pml);
+                                     qscale, po, pml, fm);
             return;
         }
     }
     launch_partial<KV, D, 4>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, qscale,
-                             po, pml);
+                             po, pml, fm);
 }
 
 // n_tok query tokens against a cache of kv_len positions that already holds them: token t
@@ -479,9 +524,21 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     const int64_t kv_len0 = kv_len - n_tok;
     dim3 grid(plan.splits, plan.nhg, Hkv);
+    // The merge runs inside this launch when the workspace carries ticket records for every row
+    // group; otherwise (or when asked for) it is a second launch.
+    FusedMerge fm{nullptr, nullptr, 0, 0, gate, out};
+    TicketRecords *tk = ws.tickets;
+    const size_t groups = (size_t)Hkv * plan.nhg;
+    const bool fused = !partial_only && !ws.separate_merge && tk && tk->dev && groups <= tk->cap;
+    if (fused) {
+        fm.rec = tk->dev + (size_t)tk->cur * tk->cap;
+        fm.zero = tk->dev + (size_t)(tk->cur ^ 1) * tk->cap;
+        fm.n_zero = (int)tk->used[tk->cur ^ 1];
+        fm.wait = ws.merge_wait;
+    }
 #define MFA_LAUNCH(KV, DD)                                                                          \
     launch_partial_w<KV, DD>(plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, Hq, n_tok, \
-                             kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml)
+                             kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml, fm)
     if (kv_dtype == MFA_KV_BF16) {
         if (D == 64) MFA_LAUNCH(uint16_t, 64);
         else if (D == 128) MFA_LAUNCH(uint16_t, 128);
@@ -493,6 +550,12 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
     }
 #undef MFA_LAUNCH
     MFA_HIP(hipGetLastError());
+    if (fused) {   // this set is in use now, the other one is clean again
+        tk->used[tk->cur] = groups;
+        tk->used[tk->cur ^ 1] = 0;
+        tk->cur ^= 1;
+        return MFA_OK;
+    }
     if (partial_only) return MFA_OK;
     launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, n_tok, gate, out);
     MFA_HIP(hipGetLastError());

@@ -138,6 +138,11 @@ class Ctx:
     def set_num_splits(self, n: int):
         _chk(self.lib.mfa_set_num_splits(self.h, n), "mfa_set_num_splits")
 
+    def set_merge(self, in_launch: bool = False, helper_polls: int = -1):
+        """How split-K partials are combined: as a second launch (default) or inside the
+        attention launch; helper_polls bounds how long early workgroups look on (-1: default)."""
+        _chk(self.lib.mfa_set_merge(self.h, int(in_launch), helper_polls), "mfa_set_merge")
+
     # ---- full attention -------------------------------------------------------
     def kv_append(self, layer, k, v):
         k, v = _f32(k, self.cfg.kv_dim, "k"), _f32(v, self.cfg.kv_dim, "v")

@@ -42,6 +42,7 @@ SIGNATURES = {
     "mfa_set_linear_weights": (C.c_int, [vp, i32, u16p, f32p, u16p, u16p]),
     "mfa_set_num_splits": (C.c_int, [vp, i32]),
     "mfa_set_partial_only": (C.c_int, [vp, i32]),
+    "mfa_set_merge": (C.c_int, [vp, i32, i32]),
     "mfa_kv_append": (C.c_int, [vp, i32, f32p, f32p]),
     "mfa_kv_append_dev": (C.c_int, [vp, i32, f32p, f32p]),
     "mfa_kv_len": (i32, [vp, i32]),

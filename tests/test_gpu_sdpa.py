@@ -158,6 +158,33 @@ def test_merge_of_several_hundred_splits(mfa, oracle, bf16):
         assert max(seen) > 256
 
 
+@pytest.mark.parametrize("Hq,Hkv,d,L,bf16", [(32, 2, 256, 9000, True), (32, 2, 256, 3000, False),
+                                             (32, 4, 128, 4096, False), (16, 2, 128, 5000, True),
+                                             (8, 8, 64, 2500, False), (40, 2, 128, 3100, True)])
+def test_merge_inside_the_launch_equals_the_separate_launch(mfa, oracle, Hq, Hkv, d, L, bf16):
+    """The same partials combined by a second launch, by the workgroup that arrives last alone
+    (no helper waits), with the default helper wait and with a long one: bit-identical results,
+    at split counts that take the few-split path (3, 8, 12, 16), the many-split path with helpers
+    (17, 20, 40, 64, 130, 300) and the default plan; several calls in a row, so that both sets of
+    ticket records are used and cleared in turn."""
+    q, g, k, v = sdpa_random_inputs(900 + L, Hq, Hkv, d, L, bf16=bf16)
+    kf = oracle.bf16_to_f32(k) if bf16 else k
+    vf = oracle.bf16_to_f32(v) if bf16 else v
+    ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+    with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
+              head_dim=d, kv_capacity=L, kv_dtype=1 if bf16 else 0) as c:
+        c.kv_import(0, kf, vf)
+        for ns in (0, 3, 8, 12, 16, 17, 20, 40, 64, 130, 300):
+            c.set_num_splits(ns)
+            c.set_merge(in_launch=False)
+            base = c.sdpa_decode(0, q, g)
+            assert rel_err(base, ref) <= (1e-4 if bf16 else TOL_F32), ns
+            for polls in (0, -1, 4000, 0, -1):
+                c.set_merge(in_launch=True, helper_polls=polls)
+                out = c.sdpa_decode(0, q, g)
+                assert np.array_equal(out, base), (ns, polls)
+
+
 def test_config3_full_size_bf16(mfa, oracle):
     """The 32K bf16 decode shape (the headline workload): 32 Q / 2 KV heads, d=256, L=32768, bf16 K/V, via bulk import."""
     Hq, Hkv, d, L = 32, 2, 256, 32768
