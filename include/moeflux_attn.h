@@ -137,6 +137,20 @@ int mfa_sdpa_decode(mfa_ctx *ctx, int32_t layer, const float *q, const float *q_
 int mfa_sdpa_decode_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev,
                         const float *q_gate_dev, float *out_dev);
 
+/* mfa_sdpa_decode_dev for callers that cannot allocate.  It has no counterpart in the
+ * reference: it is for code under HIP graph capture, tight serving loops and harnesses that
+ * forbid hipMalloc.  Same arguments, same kernels, same results bit for bit; the split-K
+ * partials go into a file-scope device array of the library (8.25 MiB per GPU, held until the
+ * process ends; its address is looked up when the first context on a device is created)
+ * instead of the context's workspace, and the call makes no hipMalloc, hipFree or other
+ * allocating call whatever the cache length.  MFA_ERR_INVALID, with nothing launched, when the
+ * split plan's partials exceed the array (more than 2 Mi f32 of partial rows: for instance
+ * more than 128 splits of 2 kv-head groups at head_dim 256).  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two contexts, two streams) race; calls on one context
+ * are ordered by its stream.  Nothing in the array has to be cleared between calls. */
+int mfa_sdpa_decode_static_dev(mfa_ctx *ctx, int32_t layer, const float *q_dev,
+                               const float *q_gate_dev, float *out_dev);
+
 /* ---- the projections either side of the attention core ------------------------ */
 
 /* One 4-bit group-64 affine dequantising matrix-vector product, all pointers on

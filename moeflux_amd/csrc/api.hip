@@ -184,6 +184,7 @@ static int create(const mfa_config *cfg, Ctx **out) {
     hipDeviceProp_t prop;
     MFA_HIP(hipGetDeviceProperties(&prop, c->device));
     c->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    MFA_TRY(static_scratch_init(c->device));
     MFA_HIP(hipStreamCreate(&c->stream));
     MFA_HIP(hipEventCreate(&c->ev0));
     MFA_HIP(hipEventCreate(&c->ev1));

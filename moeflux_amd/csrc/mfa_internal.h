@@ -277,6 +277,10 @@ int launch_plain_copy(hipStream_t stream, void *dst, const void *src, size_t nby
 // A launch that only reads nbytes (sink: 16 bytes per workgroup, never written in practice).
 int launch_plain_read(hipStream_t stream, const void *src, size_t nbytes, int workgroups, void *sink);
 
+// sdpa_static.hip: looks up, once per device, the device address of the file-scope scratch array
+// of mfa_sdpa_decode_static_dev; `device` must be the current device.
+int static_scratch_init(int device);
+
 // checkpoint.hip
 void drop_checkpoints(Ctx *c);   // frees every stored checkpoint (reset, destroy)
 

@@ -48,6 +48,7 @@ SIGNATURES = {
     "mfa_kv_len": (i32, [vp, i32]),
     "mfa_sdpa_decode": (C.c_int, [vp, i32, f32p, f32p, f32p]),
     "mfa_sdpa_decode_dev": (C.c_int, [vp, i32, f32p, f32p, f32p]),
+    "mfa_sdpa_decode_static_dev": (C.c_int, [vp, i32, f32p, f32p, f32p]),
     "mfa_prefill_attn": (C.c_int, [vp, i32, i32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_prefill_attn_dev": (C.c_int, [vp, i32, i32, f32p, f32p, f32p, f32p, f32p]),
     "mfa_gdn_step": (C.c_int, [vp, i32, f32p, f32p, f32p, f32p, f32p]),

@@ -56,6 +56,8 @@ extern "C" {
     pub fn mfa_kv_append_dev(ctx: *mut mfa_ctx, layer: i32, k: *const f32, v: *const f32) -> c_int;
     pub fn mfa_sdpa_decode_dev(ctx: *mut mfa_ctx, layer: i32, q: *const f32, q_gate: *const f32,
         out: *mut f32) -> c_int;
+    pub fn mfa_sdpa_decode_static_dev(ctx: *mut mfa_ctx, layer: i32, q_dev: *const f32, q_gate_dev: *const f32,
+        out_dev: *mut f32) -> c_int;
     pub fn mfa_gdn_step_dev(ctx: *mut mfa_ctx, layer: i32, qkv_in: *const f32, z: *const f32,
         alpha: *const f32, beta: *const f32, out: *mut f32) -> c_int;
     pub fn mfa_token_sweep_dev(ctx: *mut mfa_ctx, full_q: *const f32, full_gate: *const f32,
