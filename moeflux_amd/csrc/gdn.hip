@@ -31,10 +31,10 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     const float *__restrict__ alpha, const float *__restrict__ beta, float *__restrict__ out) {
     constexpr int NI = DK / 32;
     constexpr int NT = DV * 8;
-    constexpr int NWAVE = NT / 64;
     constexpr int KT = KC > 0 ? KC : 1;
+    constexpr int NCONV = 2 * DK + DV;   // conv channels of a head: whole waves
+    static_assert(NCONV % 64 == 0 && DV % 64 == 0 && NCONV < NT, "conv channels and outputs fill whole waves");
     __shared__ float s_q[DK], s_k[DK], s_v[DV], s_o[DV];
-    __shared__ float s_part[NWAVE];
     __shared__ float s_gb[2];
 
     const int tid = threadIdx.x;
@@ -58,45 +58,52 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
         out += ly * Hv * DV;
     }
 
-    // Which conv channel this thread serves: the head's q, k and v channels.
-    const bool conv_thread = tid < 2 * DK + DV;
+    // Which conv channel this thread serves: the head's q, k and v channels are the first
+    // NCONV threads (whole waves); the other waves only hold state rows.
+    const bool conv_thread = tid < NCONV;
     int ch = 0;
     bool owner = true;  // q/k channels are shared by `rep` value heads; one of them rolls the ring
     if (tid < DK) { ch = kh * DK + tid; owner = (vh % rep) == 0; }
     else if (tid < 2 * DK) { ch = Hk * DK + kh * DK + (tid - DK); owner = (vh % rep) == 0; }
     else if (conv_thread) ch = 2 * Hk * DK + vh * DV + (tid - 2 * DK);
 
-    // 1. Requests in the order their data is needed (loads return in order): the small
-    //    operands of the conv, the gates and the output norm first, the state rows last,
-    //    so that the conv and the norms run while the state is still streaming in.
+    // 1. Requests.  A CU takes a wave's request for 16 bytes per lane in 16 clocks and returns
+    //    data in request order, so the few small operands the whole workgroup waits for (conv
+    //    inputs and taps; z and the norm weight) are requested by the waves that use them and
+    //    nobody else, and the barrier keeps every wave's state rows (1024 clocks of requests
+    //    at dk = dv = 128) behind them.
     float x_in = 0.f, tap[KT], wt[KT];
-    if (KC > 0) {
-        x_in = qkv_in[ch];
-        const uint2 wbits = *(const uint2 *)(conv_w + (size_t)ch * 4);  // four bf16 taps
-        wt[0] = bf16_bits_to_f32((uint16_t)(wbits.x & 0xffffu));
-        if (KC > 1) wt[1 % KT] = bf16_bits_to_f32((uint16_t)(wbits.x >> 16));
-        if (KC > 2) wt[2 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y & 0xffffu));
-        if (KC > 3) wt[3 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y >> 16));
+    float z_in = 0.f, nw_in = 0.f;
+    if (conv_thread) {
+        if (KC > 0) {
+            x_in = qkv_in[ch];
+            const uint2 wbits = *(const uint2 *)(conv_w + (size_t)ch * 4);  // four bf16 taps
+            wt[0] = bf16_bits_to_f32((uint16_t)(wbits.x & 0xffffu));
+            if (KC > 1) wt[1 % KT] = bf16_bits_to_f32((uint16_t)(wbits.x >> 16));
+            if (KC > 2) wt[2 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y & 0xffffu));
+            if (KC > 3) wt[3 % KT] = bf16_bits_to_f32((uint16_t)(wbits.y >> 16));
 #pragma unroll
-        for (int k = 0; k < KT - 1; k++) {
-            int sl = slot_new + 1 + k;
-            if (sl >= KC) sl -= KC;
-            tap[k] = conv_ring[(size_t)sl * C + ch];
+            for (int k = 0; k < KT - 1; k++) {
+                int sl = slot_new + 1 + k;
+                if (sl >= KC) sl -= KC;
+                tap[k] = conv_ring[(size_t)sl * C + ch];
+            }
+        }
+        if (tid < DV) {
+            z_in = z[(size_t)vh * DV + tid];
+            nw_in = bf16_bits_to_f32(norm_w[tid]);
         }
     }
-    const int nz = tid < DV ? tid : 0;
-    const float z_in = z[(size_t)vh * DV + nz];
-    const float nw_in = bf16_bits_to_f32(norm_w[nz]);
     const float a_log_in = a_log[vh], alpha_in = alpha[vh], beta_in = beta[vh];
     const float dt_in = bf16_bits_to_f32(dt_bias[vh]);
+    __builtin_amdgcn_s_barrier();
     float *srow = ssm + ((size_t)vh * DV + r) * DK + 4 * j;
     float4 s[NI];
 #pragma unroll
-    for (int i = 0; i < NI; i++) s[i] = *(const float4 *)(srow + 32 * i);
+    for (int i = 0; i < NI; i++) s[i] = load_f4(srow + 32 * i);
 
     // 2. depthwise conv + SiLU on this head's q, k and v channels
     //    (linear_attn.rs:132-154; taps oldest first, the new input is tap K-1).
-    float cval = 0.f;
     if (conv_thread) {
         float acc = 0.f;
         if (KC > 0) {
@@ -112,64 +119,71 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
             }
             acc = fmaf(x_in, bf16_bits_to_f32(conv_w[(size_t)ch * K + (K - 1)]), acc);
         }
-        cval = silu_f(acc);
+        const float cval = silu_f(acc);
         if (owner) conv_ring[(size_t)slot_new * C + ch] = x_in;
-        if (tid >= 2 * DK) s_v[tid - 2 * DK] = cval;
+        if (tid < DK) s_q[tid] = cval;
+        else if (tid < 2 * DK) s_k[tid - DK] = cval;
+        else s_v[tid - 2 * DK] = cval;
     }
-    // 3. per-head sum of squares of q (waves [0, DK/64)) and k (waves [DK/64, 2DK/64))
-    {
-        const float sq = (tid < 2 * DK) ? cval * cval : 0.f;
-        const float ws = group_sum<64>(sq);
-        if ((tid & 63) == 0) s_part[tid >> 6] = ws;
-    }
-    // 4. decay and beta gate (shaders.metal:1321-1326)
+    // 3. decay and beta gate (shaders.metal:1321-1326)
     if (tid == NT - 1) {
-        const float a_cap = expf(a_log_in);
-        const float sp = logf(1.0f + expf(alpha_in + dt_in));
-        s_gb[0] = expf(-a_cap * sp);
-        s_gb[1] = 1.0f / (1.0f + expf(-beta_in));
+        // One lane, and every wave waits for it: the hardware exp2 / log2 / reciprocal (1 ulp each)
+        // instead of the library routines, about 100 clocks instead of 1000.
+        const float a_cap = __expf(a_log_in);
+        const float sp = __logf(1.0f + __expf(alpha_in + dt_in));   // the reference's plain softplus
+        s_gb[0] = __expf(-a_cap * sp);
+        s_gb[1] = __builtin_amdgcn_rcpf(1.0f + __expf(-beta_in));
     }
+    const float og = nw_in * silu_f(z_in);   // the output's gate and weight, ready before the read-out
     __syncthreads();
-    if (tid < 2 * DK) {
-        // infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2, k *= 1/sqrt(dk)
-        const bool is_q = tid < DK;
-        float sum = 0.f;
+
+    // 4. q and k as this thread's row slice needs them, normed on the way: the 8 lanes of a row
+    //    hold all dk channels between them, so each row forms both sums of squares itself
+    //    (infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2, k *= 1/sqrt(dk)).
+    float4 kk[NI], qq[NI];
+    {
+        float sq = 0.f, sk = 0.f;
 #pragma unroll
-        for (int w = 0; w < DK / 64; w++) sum += s_part[(is_q ? 0 : DK / 64) + w];
-        const float inv_rms = 1.0f / sqrtf(sum / (float)DK + 1e-6f);
+        for (int i = 0; i < NI; i++) {
+            kk[i] = *(const float4 *)(s_k + 32 * i + 4 * j);
+            qq[i] = *(const float4 *)(s_q + 32 * i + 4 * j);
+            sq += qq[i].x * qq[i].x + qq[i].y * qq[i].y + qq[i].z * qq[i].z + qq[i].w * qq[i].w;
+            sk += kk[i].x * kk[i].x + kk[i].y * kk[i].y + kk[i].z * kk[i].z + kk[i].w * kk[i].w;
+        }
+        sq = group_sum<8>(sq);
+        sk = group_sum<8>(sk);
         const float inv_scale = 1.0f / sqrtf((float)DK);
-        float y = cval * inv_rms;
-        y *= is_q ? inv_scale * inv_scale : inv_scale;
-        if (is_q) s_q[tid] = y; else s_k[tid - DK] = y;
+        const float iq = __builtin_amdgcn_rsqf(sq / (float)DK + 1e-6f);
+        const float ik = __builtin_amdgcn_rsqf(sk / (float)DK + 1e-6f);
+        const float q2 = inv_scale * inv_scale;
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            qq[i].x = qq[i].x * iq * q2; qq[i].y = qq[i].y * iq * q2;
+            qq[i].z = qq[i].z * iq * q2; qq[i].w = qq[i].w * iq * q2;
+            kk[i].x = kk[i].x * ik * inv_scale; kk[i].y = kk[i].y * ik * inv_scale;
+            kk[i].z = kk[i].z * ik * inv_scale; kk[i].w = kk[i].w * ik * inv_scale;
+        }
     }
-    __syncthreads();
 
     // 5. recurrence on this thread's row slice
-    float4 kk[NI], qq[NI];
-#pragma unroll
-    for (int i = 0; i < NI; i++) {
-        kk[i] = *(const float4 *)(s_k + 32 * i + 4 * j);
-        qq[i] = *(const float4 *)(s_q + 32 * i + 4 * j);
-    }
     const float o = delta_row<DK>(s, kk, qq, s_gb[0], s_gb[1], s_v[r]);
+    if (j == 0) s_o[r] = o;
 #pragma unroll
     for (int i = 0; i < NI; i++) *(float4 *)(srow + 32 * i) = s[i];
-    if (j == 0) s_o[r] = o;
     __syncthreads();
 
-    // 6. gated RMS norm over the head's dv outputs (linear_attn.rs:230-240)
-    {
-        const float x = (tid < DV) ? s_o[tid] : 0.f;
-        const float ws = group_sum<64>(x * x);
-        if ((tid & 63) == 0) s_part[tid >> 6] = ws;
-        __syncthreads();
-        if (tid < DV) {
-            float sum = 0.f;
+    // 6. gated RMS norm over the head's dv outputs (linear_attn.rs:230-240): each of the first
+    //    dv/64 waves forms the whole sum of squares itself (hardware reciprocal square root, 1 ulp).
+    if (tid < DV) {
+        float ss = 0.f;
 #pragma unroll
-            for (int w = 0; w < (DV + 63) / 64; w++) sum += s_part[w];
-            const float inv_rms = 1.0f / sqrtf(sum / (float)DV + eps);
-            out[(size_t)vh * DV + tid] = x * inv_rms * nw_in * silu_f(z_in);
+        for (int w = 0; w < DV / 64; w++) {
+            const float y = s_o[(tid & 63) + 64 * w];
+            ss += y * y;
         }
+        const float sum = group_sum<64>(ss);
+        const float inv_rms = __builtin_amdgcn_rsqf(sum / (float)DV + eps);
+        out[(size_t)vh * DV + tid] = s_o[tid] * inv_rms * og;
     }
 }
 
