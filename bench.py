@@ -486,43 +486,53 @@ def bench_matvec(steps, warmup, seed):
 
 def bench_prologue(steps, warmup, seed):
     """What precedes the attention core in a full-attention layer, at the headline shape (32 Q /
-    2 KV heads, head_dim 256, bf16 cache holding 32768 positions): the prologue alone (q/gate
-    split, per-head norms, rotation, cache append - one launch) and the whole layer step
-    (prologue + split-K attention + merge over the grown cache, mfa_full_attn_step_dev)."""
+    2 KV heads, head_dim 256, bf16 caches holding 32768 positions, 8 layers rotated over like the
+    headline's caches): the prologue alone (q/gate split, per-head norms, rotation, cache append -
+    one launch) and the whole layer step from the raw projections (mfa_full_attn_step_dev) in its
+    two forms: two launches (the attention launch norms and rotates its own query heads and
+    appends the token, the merge takes the token as one more split) and three (prologue,
+    attention, merge)."""
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
     lib = ffi.load()
-    Hq, Hkv, d, L = 32, 2, 256, 32768
-    n = 2 * (REPS * steps + warmup) + 8
-    ctx = Ctx(Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+    Hq, Hkv, d, L, NL = 32, 2, 256, 32768, 8
+    n = (3 * (REPS * steps + warmup) + 8 + NL - 1) // NL + 1
+    ctx = Ctx(Config(num_layers=NL, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                      kv_capacity=L + n, kv_dtype=ffi.KV_BF16))
     rng = np.random.default_rng(seed)
     kv = _bf16_bits(rng.standard_normal((L, Hkv * d), dtype=np.float32))
-    ctx.kv_import(0, kv, kv)
     w = _bf16_bits(np.ones(d, np.float32))
-    ctx.set_full_weights(0, w, w)
+    for l in range(NL):
+        ctx.kv_import(l, kv, kv)
+        ctx.set_full_weights(l, w, w)
     qp = DeviceArray.from_host(rng.standard_normal(2 * Hq * d).astype(np.float32))
     k = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
     v = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
     q, g, o = (DeviceArray((Hq * d,), np.float32, zero=True) for _ in range(3))
-    pos = [L]
+    pos = [L] * NL
 
     def pro(i):
-        if lib.mfa_attn_prologue_dev(ctx.h, 0, pos[0], qp.ptr, k.ptr, v.ptr, q.ptr, g.ptr) != 0:
+        l = i % NL
+        if lib.mfa_attn_prologue_dev(ctx.h, l, pos[l], qp.ptr, k.ptr, v.ptr, q.ptr, g.ptr) != 0:
             raise RuntimeError(ffi.last_error())
-        pos[0] += 1
+        pos[l] += 1
 
     def full(i):
-        if lib.mfa_full_attn_step_dev(ctx.h, 0, pos[0], qp.ptr, k.ptr, v.ptr, o.ptr) != 0:
+        l = i % NL
+        if lib.mfa_full_attn_step_dev(ctx.h, l, pos[l], qp.ptr, k.ptr, v.ptr, o.ptr) != 0:
             raise RuntimeError(ffi.last_error())
-        pos[0] += 1
+        pos[l] += 1
 
     _, pro_ms = _timed(ctx, lib, pro, steps, warmup)
-    _, full_ms = _timed(ctx, lib, full, steps, warmup)
+    lib.mfa_set_step_launches(ctx.h, 3)
+    _, full3_ms = _timed(ctx, lib, full, steps, warmup)
+    lib.mfa_set_step_launches(ctx.h, 2)
+    _, full2_ms = _timed(ctx, lib, full, steps, warmup)
     alg = 2 * Hq * d * 4 + 2 * Hkv * d * 4 + 2 * Hq * d * 4 + 2 * Hkv * d * 2
-    res = {"shape": "32 Q / 2 KV heads, head_dim 256, bf16 cache, kv_len 32768 and growing",
+    res = {"shape": "32 Q / 2 KV heads, head_dim 256, bf16 caches of 32768 positions and growing, 8 layers rotated over",
            "prologue_us_per_call": pro_ms * 1e3, "prologue_algorithmic_bytes": alg,
-           "full_attn_step_us_per_call": full_ms * 1e3, "launches_per_full_step": 3}
+           "full_attn_step_us_per_call": full2_ms * 1e3, "launches_per_full_step": 2,
+           "full_attn_step_three_launches_us_per_call": full3_ms * 1e3}
     ctx.close()
     for a in (qp, k, v, q, g, o):
         a.free()

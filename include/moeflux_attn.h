@@ -249,6 +249,12 @@ int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_
                        const float *k, const float *v, float *out);
 int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
                            const float *k_dev, const float *v_dev, float *out_dev);
+/* How many launches mfa_full_attn_step makes; no counterpart in the reference and no result
+ * depends on it beyond rounding.  2 (default, where rotary_dim / 2 is a multiple of 8 channels
+ * for a bf16 cache, 4 for f32): the attention launch norms and rotates its own query heads from
+ * q_proj_out, attends to the positions the cache already holds, and scores and appends the new
+ * token; the merge launch takes the token as one more split.  3: prologue, attention, merge. */
+int mfa_set_step_launches(mfa_ctx *ctx, int32_t launches);
 /* The same for a chunk of T prompt tokens at positions pos0 .. pos0+T-1 (the token
  * loop of eval_prompt, riir/mod.rs:1196-1214, over full_attn_layer_forward): every
  * token's q and k are normed and rotated at its own position, the T rows are

@@ -223,6 +223,9 @@ static int create(const mfa_config *cfg, Ctx **out) {
         char *qg;
         MFA_TRY(slab_alloc(c, 2 * (size_t)cfg->num_attn_heads * cfg->head_dim * sizeof(float), &qg));
         c->qg_stage = (float *)qg;
+        char *sc;
+        MFA_TRY(slab_alloc(c, (size_t)cfg->num_kv_heads * ((cfg->num_attn_heads / cfg->num_kv_heads + 15) / 16) * 16 * sizeof(float), &sc));
+        c->step_score = (float *)sc;
         // variants.rs:245-250, 369: a quarter of the head is rotated, theta = 1e7
         MFA_TRY(set_rope(c, 1.0e7f, cfg->head_dim / 4));
         int splits = sdpa_pick_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
@@ -505,6 +508,14 @@ int mfa_set_merge(mfa_ctx *ctx, int32_t in_launch, int32_t helper_polls) {
     return MFA_OK;
 }
 
+int mfa_set_step_launches(mfa_ctx *ctx, int32_t launches) {
+    Ctx *c = as_ctx(ctx);
+    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
+    if (launches != 2 && launches != 3) return fail(MFA_ERR_INVALID, "step launches must be 2 or 3 (got %d)", launches);
+    c->step_launches = launches;
+    return MFA_OK;
+}
+
 int mfa_set_partial_only(mfa_ctx *ctx, int32_t on) {
     Ctx *c = as_ctx(ctx);
     if (!c) return fail(MFA_ERR_INVALID, "NULL context");
@@ -605,6 +616,34 @@ static int prologue_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_proj, 
     return MFA_OK;
 }
 
+// One token through a full-attention layer from its raw projections.  Two launches where the
+// shape allows (and no measurement switch asks otherwise): the attention launch norms and
+// rotates its own query heads and appends the token, the merge takes the token as one more
+// split.  Otherwise three: prologue, attention, merge.
+static int full_attn_step_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_proj, const float *k, const float *v,
+                              float *out) {
+    const mfa_config &g = c->cfg;
+    const size_t qd = (size_t)c->q_dim();
+    const int32_t len0 = f->len;
+    if (c->step_launches == 2 && !c->partial_only && c->separate_merge &&
+        sdpa_step_supported(g.kv_dtype, g.num_attn_heads, g.num_kv_heads, g.head_dim, c->rotary_dim)) {
+        if (!f->norms_set) return fail(MFA_ERR_INVALID, "q/k norm weights not set (mfa_set_full_weights)");
+        if (pos < 0) return fail(MFA_ERR_INVALID, "attention prologue: pos %d < 0", pos);
+        if ((int64_t)f->len + 1 > g.kv_capacity)
+            return fail(MFA_ERR_OVERFLOW, "kv cache overflow: len %d + 1 > capacity %d", f->len, g.kv_capacity);
+        MFA_TRY(launch_sdpa_step(c->stream, g.kv_dtype, g.num_attn_heads, g.num_kv_heads, g.head_dim, f->len,
+                                 c->plane_elems, f->k, f->v, q_proj, k, v, f->q_norm, f->k_norm, c->inv_freq,
+                                 c->rotary_dim, g.rms_norm_eps, pos, c->step_score, out, workspace(c), c->num_cus,
+                                 c->forced_splits));
+        f->len += 1;
+        return MFA_OK;
+    }
+    MFA_TRY(prologue_dev(c, f, pos, q_proj, k, v, c->qg_stage, c->qg_stage + qd));
+    const int rc = sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, out);
+    if (rc != MFA_OK) rollback_append(c, f, len0);
+    return rc;
+}
+
 int mfa_attn_prologue_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out_dev,
                           const float *k_dev, const float *v_dev, float *q_out_dev, float *q_gate_out_dev) {
     Ctx *c = as_ctx(ctx);
@@ -638,12 +677,7 @@ int mfa_full_attn_step_dev(mfa_ctx *ctx, int32_t layer, int32_t pos, const float
     FullLayer *f;
     MFA_TRY(full_layer(c, layer, &f));
     if (!q_proj_out_dev || !k_dev || !v_dev || !out_dev) return fail(MFA_ERR_INVALID, "NULL argument");
-    const size_t qd = (size_t)c->q_dim();
-    const int32_t len0 = f->len;
-    MFA_TRY(prologue_dev(c, f, pos, q_proj_out_dev, k_dev, v_dev, c->qg_stage, c->qg_stage + qd));
-    const int rc = sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, out_dev);
-    if (rc != MFA_OK) rollback_append(c, f, len0);
-    return rc;
+    return full_attn_step_dev(c, f, pos, q_proj_out_dev, k_dev, v_dev, out_dev);
 }
 
 int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_proj_out, const float *k,
@@ -658,13 +692,7 @@ int mfa_full_attn_step(mfa_ctx *ctx, int32_t layer, int32_t pos, const float *q_
     MFA_TRY(h2d(c, qp, q_proj_out, 2 * qd * 4));
     MFA_TRY(h2d(c, kk, k, kd * 4));
     MFA_TRY(h2d(c, vv, v, kd * 4));
-    const int32_t len0 = f->len;
-    MFA_TRY(prologue_dev(c, f, pos, qp, kk, vv, c->qg_stage, c->qg_stage + qd));
-    const int rc = sdpa_decode_dev(c, f, c->qg_stage, c->qg_stage + qd, oo);
-    if (rc != MFA_OK) {
-        rollback_append(c, f, len0);
-        return rc;
-    }
+    MFA_TRY(full_attn_step_dev(c, f, pos, qp, kk, vv, oo));
     return d2h_sync(c, out, oo, qd * 4);
 }
 

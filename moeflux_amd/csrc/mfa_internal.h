@@ -158,6 +158,8 @@ struct Ctx {
     float *inv_freq = nullptr;
     int32_t rotary_dim = 0;
     float *qg_stage = nullptr;   // q and gate of mfa_full_attn_step, 2 * q_dim floats
+    float *step_score = nullptr; // the new token's score per query row of the two-launch attention step
+    int32_t step_launches = 2;   // launches of mfa_full_attn_step: 2 (prologue inside the attention launch) or 3
     float *qg_chunk = nullptr;   // the same for a chunk of tokens (mfa_prefill_full_attn), grown on demand
     size_t qg_chunk_elems = 0;
     int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
@@ -224,6 +226,15 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
                 int forced_splits, int partial_only = 0);
+// One decode token of a full-attention layer from its raw projections in two launches (the
+// attention launch norms and rotates the query itself and appends the token; the merge takes
+// the token as one more split).  len0: cache length before the call.
+bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim);
+int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t len0, size_t plane_elems,
+                     void *k_tiled, void *v_tiled, const float *q_proj, const float *k_in, const float *v_in,
+                     const uint16_t *q_norm, const uint16_t *k_norm, const float *inv_freq, int rotary_dim,
+                     float eps, int32_t pos, float *new_score, float *out, const SdpaWorkspace &ws, int num_cus,
+                     int forced_splits);
 // Log-sum-exp merge of partials laid out [kv head][16-row group][split][16][D] (+ (max, sum) per row),
 // normalisation, and the sigmoid gate when `gate` is not null.  out, gate: [n_tok, Hq*D].
 int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,

@@ -36,6 +36,7 @@
 //   looked on for a bounded time) combines the group's partials.  No workgroup ever
 //   depends on another one making progress.  sdpa_merge_kernel / sdpa_merge_few_kernel
 //   are the same merge as a launch of its own (the latent-cache attention uses them).
+#include "attn_prologue.h"
 #include "sdpa_merge.h"
 
 namespace mfa {
@@ -69,15 +70,128 @@ struct FusedMerge {
     float *out;
 };
 
+// The attention prologue of one decode token inside the split-K launch
+// (full_attn_forward.rs:238-323: q/gate split, per-head RMS norms of q and k, rotation of the
+// first rotary_dim channels, cache append).  The launch attends to the positions the cache held
+// before the token; the token's own score and value enter in the merge as one more split.
+struct StepPrologue {
+    const float *q_proj;       // [Hq][2][D]: q_h then gate_h
+    const float *k_in, *v_in;  // [Hkv * D] projections of the new token
+    const uint16_t *q_norm, *k_norm;
+    const float *inv_freq;     // 1 / theta^(2i/rotary_dim), i < rotary_dim / 2
+    int rotary_dim;
+    float eps;
+    int pos;                   // rotation position of the token
+    int64_t cache_pos;         // where its row goes: the cache length before the call
+    float *new_score;          // [kv head][row group][16]: q . k_new in log2 units
+    void *k_tiled, *v_tiled;   // the planes, to append to
+};
+
+// The query operands of the workgroup's 16 rows from the raw q projection: a group of
+// LPH = D / EPS lanes serves one head, lane j its channels [EPS j, EPS j + EPS), which is exactly
+// operand slot (k-step j / 4, lane group j % 4, row n).  Norm and rotation stay inside the
+// group (sums and partners by lane exchange); the arithmetic is that of attn_prologue_kernel.
+// request() only asks for the operands (all loads unconditional, so the cache requests that
+// follow can be counted apart from them); finish() does the arithmetic.  With `with_new` every
+// group also forms the new token's normed, rotated key (each the same one) and its score
+// against the group's head, and group 0 of row group 0 appends the token's key and value row.
+template <typename KV, int D, int NT> struct StepQuery {
+    using W = Wave<KV, D>;
+    static constexpr int EPS = sizeof(KV) == 2 ? 8 : 4;
+    static constexpr int LPH = D / EPS;
+    static constexpr int NQ = (W::QSLOTS + NT - 1) / NT;
+    static_assert(LPH <= 64 && W::QSLOTS == 16 * LPH, "a head's lanes fit a wave");
+    float qraw[NQ][EPS], kraw[EPS], vraw[EPS], wq[EPS], wk[EPS], freq;
+
+    __device__ inline void request(const StepPrologue &sp, const RowGroup &rows) {
+        const int j = threadIdx.x % LPH, c0 = EPS * j;
+        freq = HeadRotor<EPS, D>::table_request(sp.inv_freq, sp.rotary_dim);
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            int v = threadIdx.x + i * NT;
+            if (v >= W::QSLOTS) v = W::QSLOTS - 1;
+            const int n = v / LPH;
+            const float *p = sp.q_proj + (rows.valid(n) ? rows.q_row(n) : 0) * 2 * D + c0;
+#pragma unroll
+            for (int e = 0; e < EPS; e += 4) {
+                const float4 t = load_f4(p + e);
+                qraw[i][e] = t.x; qraw[i][e + 1] = t.y; qraw[i][e + 2] = t.z; qraw[i][e + 3] = t.w;
+            }
+        }
+        const float *pk = sp.k_in + (size_t)rows.kvh * D + c0, *pv = sp.v_in + (size_t)rows.kvh * D + c0;
+#pragma unroll
+        for (int e = 0; e < EPS; e += 4) {
+            const float4 a = load_f4(pk + e), b = load_f4(pv + e);
+            kraw[e] = a.x; kraw[e + 1] = a.y; kraw[e + 2] = a.z; kraw[e + 3] = a.w;
+            vraw[e] = b.x; vraw[e + 1] = b.y; vraw[e + 2] = b.z; vraw[e + 3] = b.w;
+        }
+        {   // EPS bf16 weights each: one 8- or 16-byte request per array
+            typedef unsigned short __attribute__((ext_vector_type(EPS))) wvec;
+            const wvec a = *reinterpret_cast<const wvec *>(sp.q_norm + c0), b = *reinterpret_cast<const wvec *>(sp.k_norm + c0);
+#pragma unroll
+            for (int e = 0; e < EPS; e++) {
+                wq[e] = bf16_bits_to_f32(a[e]);
+                wk[e] = bf16_bits_to_f32(b[e]);
+            }
+        }
+    }
+
+    // `tab`: the workgroup's (cos, sin) table (HeadRotor::table), complete before this call
+    __device__ inline void finish(const StepPrologue &sp, const RowGroup &rows, float qscale, size_t plane_elems,
+                                  bool with_new, uint4 *qlds, int nhg, const float2 *tab) {
+        const int j = threadIdx.x % LPH, c0 = EPS * j;
+        HeadRotor<EPS, D> hr;
+        hr.init(j, sp.rotary_dim, tab);
+        auto norm_rotate = [&](float (&x)[EPS], const float (&w)[EPS]) { hr.apply(x, w, sp.eps); };
+        float knew[EPS];
+        if (with_new) {   // uniform over the workgroup
+            norm_rotate(kraw, wk);
+#pragma unroll
+            for (int e = 0; e < EPS; e++) knew[e] = from_kv(to_kv<KV>(kraw[e]));   // as the cache will hold it
+        }
+#pragma unroll
+        for (int i = 0; i < NQ; i++) {
+            const int v = threadIdx.x + i * NT;
+            const bool in = v < W::QSLOTS;
+            const int n = (in ? v : W::QSLOTS - 1) / LPH;
+            const bool ok = in && rows.valid(n);
+            norm_rotate(qraw[i], wq);
+            if (with_new) {
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < EPS; e++) d = fmaf(qraw[i][e], knew[e], d);
+                d = lanes_sum<LPH>(d);
+                if (ok && j == 0) sp.new_score[((size_t)rows.kvh * nhg + rows.hg) * 16 + n] = d * qscale;
+            }
+            if (in) {
+                float4 raw[W::QRAW_F4];
+#pragma unroll
+                for (int e = 0; e < EPS; e += 4)
+                    raw[e / 4] = ok ? float4{qraw[i][e], qraw[i][e + 1], qraw[i][e + 2], qraw[i][e + 3]}
+                                    : float4{0.f, 0.f, 0.f, 0.f};
+                W::store_q_slot(qlds, raw, (j / 4) * 64 + (j % 4) * 16 + n, qscale);
+            }
+        }
+        if (with_new && rows.hg == 0 && threadIdx.x < LPH) {   // the token's row: key normed and rotated, value as it comes
+            KV *kp = (KV *)sp.k_tiled + (size_t)rows.kvh * plane_elems, *vp = (KV *)sp.v_tiled + (size_t)rows.kvh * plane_elems;
+#pragma unroll
+            for (int e = 0; e < EPS; e++) {
+                kp[KvTile<KV>::k_off(sp.cache_pos, c0 + e, D)] = to_kv<KV>(kraw[e]);
+                vp[KvTile<KV>::v_off(sp.cache_pos, c0 + e, D)] = to_kv<KV>(vraw[e]);
+            }
+        }
+    }
+};
+
 static constexpr int kFewSplits = 16;        // at most this many: merged by one workgroup in one go
 static constexpr int kMaxMergeChunks = 32;   // claim bits of a record
 
-template <typename KV, int D, int WAVES>
+template <typename KV, int D, int WAVES, bool STEP>
 __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
     const float *__restrict__ q, int hpk, int Hq, int n_tok, int64_t kv_len0,
     int blocks_per_split, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml,
-    FusedMerge fm) {
+    FusedMerge fm, StepPrologue sp) {
     using W = Wave<KV, D>;
     constexpr int NACC = W::NACC;
     constexpr int TPW = NACC / WAVES;  // output tiles owned by one wave
@@ -89,11 +203,13 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     __shared__ uint4 pbuf[WAVES][W::P_U4][64];
     __shared__ float sm[WAVES][16];
     __shared__ float sl[WAVES][16];
+    __shared__ float2 s_tab[STEP ? 128 : 1];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, hg = blockIdx.y, kvh = blockIdx.z;
-    const int nsplit = gridDim.x, nhg = gridDim.y;
+    // a decode step's launch has one more workgroup per row group, which only scores and appends the new token
+    const int nsplit = gridDim.x - (STEP ? 1 : 0), nhg = gridDim.y;
 
     const int64_t blk_elems = (int64_t)W::BLK * D;
     const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
@@ -112,6 +228,17 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
         for (int i = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; i < fm.n_zero; i += nwg)
             fm.zero[i] = 0ull;
     }
+    if (STEP && split == nsplit) {
+        // The token's own workgroup: its key normed and rotated, its score against every query
+        // row of the group, and its row appended - off the path of the workgroups that stream
+        // the cache.  It leaves no partial; the merge takes the score and the value row directly.
+        StepQuery<KV, D, WAVES * 64> sq;
+        sq.request(sp, rows);
+        HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
+        __syncthreads();
+        sq.finish(sp, rows, qscale, plane_elems, true, qlds, nhg, s_tab);
+        return;
+    }
     if (b0 >= b1) {  // a split that lies wholly beyond what this group's rows may see
         // Its rows of part_o stay unwritten: the merge gives a split whose maximum is -inf the
         // weight 0 by selection, so whatever bytes the workspace holds there never enter a sum.
@@ -127,25 +254,33 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     // compiler can count outstanding loads exactly and wait for the query without
     // waiting for the cache.
     float4 qraw[NQ][W::QRAW_F4];
+    StepQuery<KV, D, WAVES * 64> sq;
+    if (STEP) {
+        sq.request(sp, rows);
+        __builtin_amdgcn_s_barrier();
+    } else {
 #pragma unroll
-    for (int i = 0; i < NQ; i++) {
-        int slot = threadIdx.x + i * WAVES * 64;
-        if (slot >= W::QSLOTS) slot = W::QSLOTS - 1;
-        W::load_q_slot(qraw[i], q, slot, rows);
+        for (int i = 0; i < NQ; i++) {
+            int slot = threadIdx.x + i * WAVES * 64;
+            if (slot >= W::QSLOTS) slot = W::QSLOTS - 1;
+            W::load_q_slot(qraw[i], q, slot, rows);
+        }
+        // A CU returns load data in request order across its waves: hold the bulk requests
+        // back until every wave's query request is queued, or a late wave's query would
+        // sit behind its siblings' cache blocks.
+        __builtin_amdgcn_s_barrier();
     }
-    // A CU returns load data in request order across its waves: hold the bulk requests
-    // back until every wave's query request is queued, or a late wave's query would
-    // sit behind its siblings' cache blocks.
-    __builtin_amdgcn_s_barrier();
     uint4 kreg[NLOAD];
     uint4 vreg[WAVES][TPW];
-    auto load_k =[&](int64_t sb) {
+    // loads [i0, i1) of this wave's K block of the super-block starting at sb
+    auto load_k_part = [&](int64_t sb, int i0, int i1) {
         int64_t blk = sb + wave;
         if (blk > b1 - 1) blk = b1 - 1;  // a wave without a block re-reads the last one and ignores it
         const uint4 *p = (const uint4 *)(kplane + blk * blk_elems) + lane;
 #pragma unroll
-        for (int i = 0; i < NLOAD; i++) kreg[i] = stream_load(p + i * 64);
+        for (int i = i0; i < i1; i++) kreg[i] = stream_load(p + i * 64);
     };
+    auto load_k = [&](int64_t sb) { load_k_part(sb, 0, NLOAD); };
     // V of blocks [j0, j1) of the super-block starting at sb
     auto load_v = [&](int64_t sb, int j0, int j1) {
 #pragma unroll
@@ -161,12 +296,25 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     // all of V here would keep the wave stuck in the issue stage long after its K has
     // arrived.  So only kVEarly blocks of V go out now, the rest once the scores are under way.
     constexpr int kVEarly = WAVES / 4;
-    load_k(b0);
-    load_v(b0, 0, kVEarly);
+    if (STEP) {
+        // Half of the K block is requested first: enough to keep the memory pipeline full while
+        // the first wave forms the rotation table and every wave norms and rotates its share of
+        // the query (a wave cannot compute while its requests wait for room in the queue, which
+        // the full set would do for microseconds).  The rest follows when the query is in LDS.
+        load_k_part(b0, 0, NLOAD / 2);
+        HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
+        __syncthreads();
+        sq.finish(sp, rows, qscale, plane_elems, false, qlds, nhg, s_tab);
+        load_k_part(b0, NLOAD / 2, NLOAD);
+        load_v(b0, 0, kVEarly);
+    } else {
+        load_k(b0);
+        load_v(b0, 0, kVEarly);
 #pragma unroll
-    for (int i = 0; i < NQ; i++) {
-        const int slot = threadIdx.x + i * WAVES * 64;
-        if (slot < W::QSLOTS) W::store_q_slot(qlds, qraw[i], slot, qscale);
+        for (int i = 0; i < NQ; i++) {
+            const int slot = threadIdx.x + i * WAVES * 64;
+            if (slot < W::QSLOTS) W::store_q_slot(qlds, qraw[i], slot, qscale);
+        }
     }
     __syncthreads();
 
@@ -284,7 +432,7 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     __shared__ float4 acc4[TEAMS][2][16][16];
     __shared__ unsigned int s_own;                   // chunks this workgroup merges (bit set), 0: none
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const MergeOut mo{fm.gate, fm.out, hpk, Hq, n_tok, D};
+    const MergeOut mo{fm.gate, fm.out, hpk, Hq, n_tok, D, D, nullptr, nullptr, 0, nhg};
     const bool few = nsplit <= kFewSplits;
     // chunks of the many-split merge: a power of two, at most one per split, at most 32, and
     // not finer than what the workgroup's teams merge in one pass
@@ -355,26 +503,37 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
             const int64_t orow = mo.row(kvh, hg * 16 + nn);
             const bool active = in && orow >= 0;
             if (span == 2)
-                merge_span<2>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team]);
+                merge_span<2>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team], D);
             else
-                merge_span<1>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team]);
+                merge_span<1>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team], D);
         }
     }
 }
 
 
+// The token a decode step has just appended, as one more split of the merge (MergeOut), and
+// where the gate rows lie.
+struct MergeExtra {
+    int gate_stride;
+    const float *new_score, *new_v;
+    int new_bf16;
+};
+
 // The same merge as a launch of its own.
 // grid (n_tok * Hq, D/64), 256 threads: one 64-output unit per workgroup.
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
-    int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out) {
+    int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out, MergeExtra ex) {
     __shared__ float4 acc4[1][16][16];
     // blockIdx.x = token * Hq + head; its row in the kv head's row list is token*hpk + head%hpk
     const int h = blockIdx.x % Hq, tok = blockIdx.x / Hq;
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
+    const MergeOut mo{gate, out, hpk, Hq, 1, D, ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
+    const int c = blockIdx.y * 64 + (threadIdx.x & 63);
     merge_span<1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate, out,
-                  threadIdx.x, acc4);
+                  threadIdx.x, acc4, ex.gate_stride, mo.token_score(kvh, hg, n),
+                  ex.new_score ? mo.token_value(kvh, c) : 0.f);
 }
 
 // Few splits (at most NS = 8 or 16, what a launch over many layers or row groups ends up
@@ -382,7 +541,7 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
 template <int NS>
 __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
-    int Hq, int nhg, int D, int n_units, const float *__restrict__ gate, float *__restrict__ out) {
+    int Hq, int nhg, int D, int n_units, const float *__restrict__ gate, float *__restrict__ out, MergeExtra ex) {
     const int lane = threadIdx.x & 63;
     const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= n_units) return;   // whole waves; there is no barrier below
@@ -391,23 +550,26 @@ __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
     const int u = n * per_row + by;   // the unit's index inside its row group
-    const MergeOut mo{gate, out, hpk, Hq, (int)(((int64_t)n_units / per_row) / Hq), D};
+    const MergeOut mo{gate, out, hpk, Hq, (int)(((int64_t)n_units / per_row) / Hq), D,
+                      ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
     merge_few_units<NS, 1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, kvh, hg, u, u + 1, mo, lane);
 }
 
 static void launch_merge_kernels(hipStream_t stream, const float *part_o, const float *part_ml, int splits, int hpk,
-                                 int Hq, int nhg, int D, int n_tok, const float *gate, float *out) {
+                                 int Hq, int nhg, int D, int n_tok, const float *gate, float *out,
+                                 const MergeExtra *extra = nullptr) {
+    const MergeExtra ex = extra ? *extra : MergeExtra{D, nullptr, nullptr, 0};
     const int n_units = n_tok * Hq * (D / 64);
     const dim3 few((n_units + 3) / 4);
     if (splits <= 8)
         hipLaunchKernelGGL((sdpa_merge_few_kernel<8>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
-                           n_units, gate, out);
+                           n_units, gate, out, ex);
     else if (splits <= 16)
         hipLaunchKernelGGL((sdpa_merge_few_kernel<16>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
-                           n_units, gate, out);
+                           n_units, gate, out, ex);
     else
         hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, part_o, part_ml, splits, hpk,
-                           Hq, nhg, D, gate, out);
+                           Hq, nhg, D, gate, out, ex);
 }
 
 int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,
@@ -474,28 +636,94 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok) {
     return (size_t)Hkv * nhg * splits * 32;
 }
 
-template <typename KV, int D, int WAVES>
+template <typename KV, int D, int WAVES, bool STEP>
 static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
                            size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                           int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm) {
-    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES>), grid, dim3(WAVES * 64), 0, stream,
+                           int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
+                           const StepPrologue &sp) {
+    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES, STEP>), grid, dim3(WAVES * 64), 0, stream,
                        (const KV *)k, (const KV *)v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                       qscale, po, pml, fm);
+                       qscale, po, pml, fm, sp);
 }
 
-template <typename KV, int D>
+template <typename KV, int D, bool STEP>
 static void launch_partial_w(int waves, hipStream_t stream, dim3 grid, const void *k, const void *v,
                              size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                             int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm) {
+                             int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
+                             const StepPrologue &sp) {
     if constexpr (D >= 128) {
         if (waves == 8) {
-            launch_partial<KV, D, 8>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                                     qscale, po, pml, fm);
+            launch_partial<KV, D, 8, STEP>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
+                                           qscale, po, pml, fm, sp);
             return;
         }
     }
-    launch_partial<KV, D, 4>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, qscale,
-                             po, pml, fm);
+    launch_partial<KV, D, 4, STEP>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, qscale,
+                                   po, pml, fm, sp);
+}
+
+// dtype and width dispatch of the split-K launch
+template <bool STEP>
+static void launch_partial_any(int kv_dtype, int D, int waves, hipStream_t stream, dim3 grid, const void *k,
+                               const void *v, size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
+                               int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
+                               const StepPrologue &sp) {
+#define MFA_LAUNCH(KV, DD)                                                                                  \
+    launch_partial_w<KV, DD, STEP>(waves, stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, \
+                                   qscale, po, pml, fm, sp)
+    if (kv_dtype == MFA_KV_BF16) {
+        if (D == 64) MFA_LAUNCH(uint16_t, 64);
+        else if (D == 128) MFA_LAUNCH(uint16_t, 128);
+        else MFA_LAUNCH(uint16_t, 256);
+    } else {
+        if (D == 64) MFA_LAUNCH(float, 64);
+        else if (D == 128) MFA_LAUNCH(float, 128);
+        else MFA_LAUNCH(float, 256);
+    }
+#undef MFA_LAUNCH
+}
+
+bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim) {
+    if (!sdpa_shape_supported(kv_dtype, D) || Hq % Hkv != 0) return false;
+    return head_rotor_applies(kv_dtype, D, rotary_dim);
+}
+
+// One decode token of a full-attention layer from its raw projections in two launches: the
+// split-K launch norms and rotates the query heads itself, attends to the len0 positions the
+// cache holds, and its first workgroups score and append the token; the merge adds the token as
+// one more split.  out: [Hq * D].
+int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t len0, size_t plane_elems,
+                     void *k_tiled, void *v_tiled, const float *q_proj, const float *k_in, const float *v_in,
+                     const uint16_t *q_norm, const uint16_t *k_norm, const float *inv_freq, int rotary_dim,
+                     float eps, int32_t pos, float *new_score, float *out, const SdpaWorkspace &ws, int num_cus,
+                     int forced_splits) {
+    if (!sdpa_step_supported(kv_dtype, Hq, Hkv, D, rotary_dim))
+        return fail(MFA_ERR_SHAPE, "attention step: shape not supported by the two-launch form");
+    if (len0 < 0 || pos < 0) return fail(MFA_ERR_INVALID, "attention step: negative position");
+    const int hpk = Hq / Hkv;
+    // the token's workgroups (one per row group and kv head) take CUs of their own
+    const int token_wgs = Hkv * ((hpk + 15) / 16);
+    if (num_cus > 2 * token_wgs) num_cus -= token_wgs;
+    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits);
+    while (forced_splits <= 0 && plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, 1) > ws.part_o_elems ||
+                                                     sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, 1) > ws.part_ml_elems))
+        plan = plan_splits(kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, (plan.splits + 1) / 2);
+    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, 1) > ws.part_o_elems ||
+        sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, 1) > ws.part_ml_elems)
+        return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
+    const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
+    const FusedMerge fm{nullptr, nullptr, 0, 0, nullptr, nullptr};
+    const StepPrologue sp{q_proj, k_in, v_in, q_norm, k_norm, inv_freq, rotary_dim, eps, pos, len0, new_score,
+                          k_tiled, v_tiled};
+    // rows see positions [0, len0): one token whose own position is not in the cache yet
+    launch_partial_any<true>(kv_dtype, D, plan.waves, stream, dim3(plan.splits + 1, plan.nhg, Hkv), k_tiled, v_tiled,
+                             plane_elems, nullptr, hpk, Hq, 1, len0 - 1, (int)plan.bps, qscale, ws.part_o, ws.part_ml,
+                             fm, sp);
+    MFA_HIP(hipGetLastError());
+    const MergeExtra ex{2 * D, new_score, v_in, kv_dtype == MFA_KV_BF16 ? 1 : 0};
+    launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, 1, q_proj + D, out, &ex);
+    MFA_HIP(hipGetLastError());
+    return MFA_OK;
 }
 
 // n_tok query tokens against a cache of kv_len positions that already holds them: token t
@@ -536,19 +764,8 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
         fm.n_zero = (int)tk->used[tk->cur ^ 1];
         fm.wait = ws.merge_wait;
     }
-#define MFA_LAUNCH(KV, DD)                                                                          \
-    launch_partial_w<KV, DD>(plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, Hq, n_tok, \
-                             kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml, fm)
-    if (kv_dtype == MFA_KV_BF16) {
-        if (D == 64) MFA_LAUNCH(uint16_t, 64);
-        else if (D == 128) MFA_LAUNCH(uint16_t, 128);
-        else MFA_LAUNCH(uint16_t, 256);
-    } else {
-        if (D == 64) MFA_LAUNCH(float, 64);
-        else if (D == 128) MFA_LAUNCH(float, 128);
-        else MFA_LAUNCH(float, 256);
-    }
-#undef MFA_LAUNCH
+    launch_partial_any<false>(kv_dtype, D, plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, Hq, n_tok,
+                              kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml, fm, StepPrologue{});
     MFA_HIP(hipGetLastError());
     if (fused) {   // this set is in use now, the other one is clean again
         tk->used[tk->cur] = groups;

@@ -21,6 +21,19 @@ struct MergeOut {
     const float *gate;   // may be null: no gate
     float *out;
     int hpk, Hq, n_tok, D;
+    int gate_stride;     // floats between the gate rows of consecutive heads (D, or 2 D inside a q projection)
+    // One more split that is a single position, the token a decode step has just appended:
+    // its score per row (log2 units, [kv head][row group][16]) and its value row ([Hkv * D] as
+    // projected; rounded here as the cache holds it).  Null: none.
+    const float *new_score, *new_v;
+    int new_bf16, nhg;
+    __device__ float token_score(int kvh, int hg, int n) const {
+        return new_score ? new_score[((size_t)kvh * nhg + hg) * 16 + n] : -__builtin_huge_valf();
+    }
+    __device__ float token_value(int kvh, int c) const {
+        const float v = new_v[(size_t)kvh * D + c];
+        return new_bf16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : v;
+    }
     // row rr of kv head kvh's row list (token rr / hpk, head rr % hpk of the group) -> row of out, or -1
     __device__ int64_t row(int kvh, int rr) const {
         if (rr >= n_tok * hpk) return -1;
@@ -41,7 +54,8 @@ static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 // Called by whole workgroups with a uniform `active` per team; contains two workgroup barriers.
 template <int NU, typename Reader>
 __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool active, int n, int c0, int64_t orow,
-                                  const float *gate, float *out, int ttid, float4 (*acc4)[16][16]) {
+                                  const float *gate, float *out, int ttid, float4 (*acc4)[16][16],
+                                  int gate_stride, float tok_score = -__builtin_huge_valf(), float tok_value = 0.f) {
     constexpr int R = kMergeRows / NU;
     const int lane = ttid & 63, dl = ttid & 15, sg = ttid >> 4;
     // split s of row n: maximum at statistic 32 s + n, sum at 32 s + n + 16
@@ -65,19 +79,19 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
             rows[u][r] = ok ? rd.row4((s * 16 + n) * D + c0 + 64 * u + dl * 4) : float4{0.f, 0.f, 0.f, 0.f};
     }
     const bool writer = active && ttid < 64 * NU;
-    const float gt_in = (gate && writer) ? gate[orow * D + c0 + ttid] : 0.f;
+    const float gt_in = (gate && writer) ? gate[orow * gate_stride + c0 + ttid] : 0.f;
 
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
     if (active)
         for (int s = lane + 256; s < nsplit; s += 64) m = fmaxf(m, rd.stat(s * 32 + n));
-    const float M = wave_max(m);
+    const float M = fmaxf(wave_max(m), tok_score);
     auto weight = [&](float ms_) { return (ms_ == neg_inf()) ? 0.f : fast_exp2(ms_ - M); };
     float den = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; r++) den += weight(ms[r]) * ls[r];
     if (active)
         for (int s = lane + 256; s < nsplit; s += 64) den += weight(rd.stat(s * 32 + n)) * rd.stat(s * 32 + n + 16);
-    den = group_sum<64>(den);
+    den = group_sum<64>(den) + weight(tok_score);   // the single position's sum is 1
 
     float4 acc[NU];
 #pragma unroll
@@ -113,6 +127,7 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
         float sum = 0.f;
 #pragma unroll
         for (int x = 0; x < 16; x++) sum += ((const float *)&acc4[u][x][ql])[qc];
+        sum += weight(tok_score) * tok_value;
         out[orow * D + c0 + ttid] = (sum / den) * merge_gate(gate, gt_in);
     }
     __syncthreads();   // acc4 may be written again by the next call
@@ -127,7 +142,7 @@ __device__ inline void merge_few_units(const Reader &rd, int nsplit, int kvh, in
                                        const MergeOut &mo, int lane) {
     const int D = mo.D, per_row = D / 64;
     const int sl = lane < nsplit ? lane : nsplit - 1;
-    float m_in[UPW], l_in[UPW], gt_in[UPW], rows[UPW][NS];
+    float m_in[UPW], l_in[UPW], gt_in[UPW], ts_in[UPW], tv_in[UPW], rows[UPW][NS];
     int64_t orow[UPW];
     int ch[UPW];
 #pragma unroll
@@ -141,15 +156,18 @@ __device__ inline void merge_few_units(const Reader &rd, int nsplit, int kvh, in
         l_in[i] = rd.stat(sl * 32 + n + 16);
 #pragma unroll
         for (int s = 0; s < NS; s++) rows[i][s] = rd.row1(((s < nsplit ? s : nsplit - 1) * 16 + n) * D + ch[i]);
-        gt_in[i] = (mo.gate && orow[i] >= 0) ? mo.gate[orow[i] * D + ch[i]] : 0.f;
+        gt_in[i] = (mo.gate && orow[i] >= 0) ? mo.gate[orow[i] * mo.gate_stride + ch[i]] : 0.f;
+        ts_in[i] = mo.token_score(kvh, hg, n);
+        tv_in[i] = mo.new_score ? mo.token_value(kvh, ch[i]) : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < UPW; i++) {
         const float ms = lane < nsplit ? m_in[i] : neg_inf();
-        const float M = wave_max(ms);
+        const float M = fmaxf(wave_max(ms), ts_in[i]);
         const float w = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
-        const float den = group_sum<64>(w * (lane < nsplit ? l_in[i] : 0.f));
-        float acc = 0.f;
+        const float wt = (ts_in[i] == neg_inf()) ? 0.f : fast_exp2(ts_in[i] - M);
+        const float den = group_sum<64>(w * (lane < nsplit ? l_in[i] : 0.f)) + wt;
+        float acc = wt * tv_in[i];
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             const float ws = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), s));

@@ -143,6 +143,10 @@ class Ctx:
         attention launch; helper_polls bounds how long early workgroups look on (-1: default)."""
         _chk(self.lib.mfa_set_merge(self.h, int(in_launch), helper_polls), "mfa_set_merge")
 
+    def set_step_launches(self, launches: int):
+        """Launches of full_attn_step: 2 (prologue inside the attention launch) or 3."""
+        _chk(self.lib.mfa_set_step_launches(self.h, launches), "mfa_set_step_launches")
+
     # ---- full attention -------------------------------------------------------
     def kv_append(self, layer, k, v):
         k, v = _f32(k, self.cfg.kv_dim, "k"), _f32(v, self.cfg.kv_dim, "v")

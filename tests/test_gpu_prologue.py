@@ -153,3 +153,71 @@ def test_prologue_errors(mfa):
         with pytest.raises(MfaError):
             c.attn_prologue(0, 1, z, kv, kv)        # cache full (full_attn_forward.rs:283-288)
         assert c.kv_len(0) == 1
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("Hq,Hkv,d,L0", [(32, 2, 256, 0), (32, 2, 256, 1000), (32, 2, 256, 9000), (32, 4, 128, 4100),
+                                         (8, 2, 64, 33), (16, 1, 128, 300), (4, 4, 64, 17), (40, 2, 64, 70)])
+def test_two_launch_step_equals_three_launch_step(mfa, oracle, bf16, Hq, Hkv, d, L0):
+    """A decode step whose attention launch norms and rotates its own query heads and whose merge
+    takes the new token as one more split, against the prologue / attention / merge chain: the same
+    cache rows bit for bit, the same outputs to the tolerance, and the oracle's composition
+    (full_attn_forward.rs:234-389) for every step; from an empty cache, across a block edge, with
+    16 and more than 16 query heads per kv head."""
+    rng, qn, kn = _case(L0 + d + Hq, Hq, Hkv, d)
+    steps = 3
+    k0 = rng.standard_normal((L0, Hkv * d)).astype(np.float32)
+    v0 = rng.standard_normal((L0, Hkv * d)).astype(np.float32)
+    if bf16:
+        k0, v0 = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k0, v0))
+    kc = np.concatenate([k0, np.zeros((steps, Hkv * d), np.float32)])
+    vc = np.concatenate([v0, np.zeros((steps, Hkv * d), np.float32)])
+    tol = 1e-4 if bf16 else TOL_F32
+    with _ctx(mfa, Hq, Hkv, d, L0 + steps, bf16=bf16) as a, _ctx(mfa, Hq, Hkv, d, L0 + steps, bf16=bf16) as b:
+        b.set_step_launches(3)
+        for c in (a, b):
+            c.set_full_weights(0, qn, kn)
+            if L0:
+                c.kv_import(0, k0, v0)
+        for t in range(steps):
+            pos = L0 + t
+            qp = rng.standard_normal(Hq * 2 * d).astype(np.float32)
+            k, v = rng.standard_normal(Hkv * d).astype(np.float32), rng.standard_normal(Hkv * d).astype(np.float32)
+            o2, o3 = a.full_attn_step(0, pos, qp, k, v), b.full_attn_step(0, pos, qp, k, v)
+            rq, rg, rk, rv = oracle.attn_prologue(pos, Hq, Hkv, d, d // 4, THETA, 1e-6, qn, kn, qp, k, v)
+            if bf16:
+                rk, rv = (oracle.bf16_to_f32(oracle.f32_to_bf16(x)) for x in (rk, rv))
+            kc[pos], vc[pos] = rk, rv
+            ref = oracle.sdpa(pos + 1, Hq, Hkv, d, rq, rg, kc[:pos + 1], vc[:pos + 1])
+            assert rel_err(o2, o3) <= tol, (t, rel_err(o2, o3))
+            assert rel_err(o2, ref) <= (2e-3 if bf16 else TOL_F32), (t, rel_err(o2, ref))
+            heads = np.abs(o2.reshape(Hq, d) - ref.reshape(Hq, d)).max(axis=1) / np.abs(ref.reshape(Hq, d)).max(axis=1)
+            assert heads.max() <= (4e-3 if bf16 else 2e-5), (t, heads.max())
+        assert a.kv_len(0) == b.kv_len(0) == L0 + steps
+        (ka, va), (kb, vb) = a.kv_export(0), b.kv_export(0)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+
+
+def test_two_launch_step_with_forced_splits_and_errors(mfa, oracle):
+    """The split count does not change the two-launch step's result beyond rounding, a full cache
+    is refused before anything is appended, and weights must be set."""
+    Hq, Hkv, d, L0 = 32, 2, 256, 700
+    from moeflux_amd import MfaError, ffi
+    rng, qn, kn = _case(3, Hq, Hkv, d)
+    k0, v0 = rng.standard_normal((L0, Hkv * d)).astype(np.float32), rng.standard_normal((L0, Hkv * d)).astype(np.float32)
+    qp = rng.standard_normal(Hq * 2 * d).astype(np.float32)
+    k, v = rng.standard_normal(Hkv * d).astype(np.float32), rng.standard_normal(Hkv * d).astype(np.float32)
+    outs = []
+    for splits in (0, 1, 3, 44):
+        with _ctx(mfa, Hq, Hkv, d, L0 + 1) as c:
+            with pytest.raises(MfaError):
+                c.full_attn_step(0, L0, qp, k, v)       # weights not set
+            c.set_full_weights(0, qn, kn)
+            c.kv_import(0, k0, v0)
+            c.set_num_splits(splits)
+            outs.append(c.full_attn_step(0, L0, qp, k, v))
+            with pytest.raises(MfaError) as e:
+                c.full_attn_step(0, L0 + 1, qp, k, v)   # the cache is full
+            assert e.value.code == ffi.ERR_OVERFLOW and c.kv_len(0) == L0 + 1
+    for o in outs[1:]:
+        assert rel_err(o, outs[0]) <= TOL_F32
