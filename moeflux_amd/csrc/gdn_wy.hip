@@ -58,12 +58,17 @@ __device__ inline wy_f32x4 load_v4(const float *p) { return *reinterpret_cast<co
 //
 // grid (Hv, blocks), one wave per 16 columns of K (DK/16 waves: two per SIMD at DK = 128, so that one
 // has matrix work while the other waits for LDS or stores a tile).
-template <int DK>
+// FUSED: the block's inputs come straight from the layer's inputs (WyInputs): what
+// gdn_chunk_pre_kernel computes for the token-by-token form is done here per (block, value head) -
+// conv + SiLU of the head's q, k and v channels, the per-token q/k norm, the decay's logarithm and
+// beta - so the chunk needs no launch and no arrays for them.  A k-head's q and k are formed by
+// each of the value heads that share it.
+template <int DK, bool FUSED>
 __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     int Hk, int Hv, int T, const float *__restrict__ qn, const float *__restrict__ kn,
     const float *__restrict__ vv, const float *__restrict__ lg, const float *__restrict__ bg,
     float *__restrict__ Wt, float *__restrict__ Qt, float *__restrict__ Ut, float *__restrict__ Mt,
-    float *__restrict__ Kt, float *__restrict__ eLc) {
+    float *__restrict__ Kt, float *__restrict__ eLc, WyInputs in) {
     constexpr int DV = DK;
     constexpr int NK = DK / 16;
     constexpr int LDK = DK + 4;  // row strides chosen so that 16-byte row reads by 8 lanes hit all banks
@@ -72,7 +77,8 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     constexpr int NTHR = 64 * NW;
     constexpr int NCT = 1;        // 16-wide column tiles of W (and of U) per wave
     __shared__ __align__(16) float sK[kC][LDK];
-    __shared__ __align__(16) float sQ[kC][LDK];  // q^, later v
+    __shared__ __align__(16) float sQ[kC][LDK];  // q^, later v (FUSED: q^ only)
+    __shared__ __align__(16) float sV[FUSED ? kC : 1][LDK];
     __shared__ __align__(16) float sA[kC][LDC];
     __shared__ __align__(16) float sT[kC][LDC];
     __shared__ __align__(16) float sL[kC], sB[kC], sCw[kC], sKd[kC];
@@ -90,12 +96,81 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     // Everything the block reads is requested here, in the order of use (loads return in the
     // order of their requests): the gates, k^ and q^, and v, which waits in registers for phase 2.
     float lg_in = 0.f, bg_in = 0.f;
+    constexpr int NLV = kC * (DV / 4) / NTHR;
+    float4 va[FUSED ? 1 : NLV];
+    if constexpr (FUSED) {
+        constexpr int NCONV = 2 * DK + DV, TT = 16;          // channels of the head; tokens per run
+        constexpr int NU = NCONV * (kC / TT) / NTHR;          // (channel, run) units per thread
+        static_assert(NCONV * (kC / TT) % NTHR == 0, "whole units per thread");
+        const int C = 2 * Hk * DK + Hv * DV;
+        float a_in = 0.f, b_in = 0.f, al_in = 0.f, dt_in = 0.f;
+        if (wave == 0 && lane < nt) {
+            a_in = in.alpha[(size_t)(t0 + lane) * Hv + vh];
+            b_in = in.beta[(size_t)(t0 + lane) * Hv + vh];
+            al_in = in.a_log[vh];
+            dt_in = bf16_bits_to_f32(in.dt_bias[vh]);
+        }
+        // conv + SiLU (linear_attn.rs:132-154) of channel c over a run of 16 tokens per unit
+#pragma unroll
+        for (int u = 0; u < NU; u++) {
+            const int unit = tid + u * NTHR, c = unit % NCONV, run = unit / NCONV;
+            const int ch = c < DK ? kh * DK + c : c < 2 * DK ? Hk * DK + kh * DK + (c - DK) : 2 * Hk * DK + vh * DV + (c - 2 * DK);
+            const int tr = t0 + TT * run;
+            int ntr = T - tr;
+            ntr = ntr < 0 ? 0 : ntr > TT ? TT : ntr;
+            float o[TT];
+            if (in.K == 4) {
+                conv_silu_run<TT, 4>(in.ring, in.qkv, in.conv_w, C, in.step_mod, tr, ntr, ch, o);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TT; i++)
+                    o[i] = i < ntr ? conv_silu(in.ring, in.qkv, in.conv_w, C, in.K, in.step_mod, tr + i, ch) : 0.f;
+            }
+            float(*dst)[LDK] = c < DK ? sQ : c < 2 * DK ? sK : sV;
+            const int cc = c < DK ? c : c < 2 * DK ? c - DK : c - 2 * DK;
+#pragma unroll
+            for (int i = 0; i < TT; i++) dst[TT * run + i][cc] = o[i];
+        }
+        if (wave == 0 && lane < nt) {
+            // shaders.metal:1321-1326; the decay enters as its logarithm
+            const float a_cap = expf(al_in);
+            const float sp = logf(1.0f + expf(a_in + dt_in));
+            lg_in = -a_cap * sp;
+            bg_in = 1.0f / (1.0f + expf(-b_in));
+        }
+        __syncthreads();
+        // per-token norm of q and k (infer.m:2655-2667: x * inv_rms, then q *= (1/sqrt(dk))^2,
+        // k *= 1/sqrt(dk)): NTHR / (2 kC) lanes per (token, q|k) row, in place
+        constexpr int LPP = NTHR / (2 * kC), EPL = DK / LPP;   // lanes per row, elements per lane
+        static_assert(LPP == 2 || LPP == 4, "lanes per normed row");
+        {
+            const int p = tid / LPP, sub = tid % LPP, tt = p % kC;
+            const bool is_q = p < kC;
+            float *row = (is_q ? sQ[tt] : sK[tt]) + EPL * sub;
+            float4 x[EPL / 4];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < EPL / 4; i++) {
+                x[i] = lds_f4(row + 4 * i);
+                ss += x[i].x * x[i].x + x[i].y * x[i].y + x[i].z * x[i].z + x[i].w * x[i].w;
+            }
+            ss = dpp_add<0xB1>(ss);
+            if (LPP == 4) ss = dpp_add<0x4E>(ss);
+            const float inv_scale = 1.0f / sqrtf((float)DK);
+            const float inv_rms = 1.0f / sqrtf(ss / (float)DK + 1e-6f);
+            const float sc = is_q ? inv_scale * inv_scale : inv_scale;
+#pragma unroll
+            for (int i = 0; i < EPL / 4; i++) {
+                float4 y = {x[i].x * inv_rms, x[i].y * inv_rms, x[i].z * inv_rms, x[i].w * inv_rms};
+                y.x *= sc; y.y *= sc; y.z *= sc; y.w *= sc;
+                *(float4 *)(row + 4 * i) = y;
+            }
+        }
+    } else {
     if (wave == 0 && lane < nt) {
         lg_in = lg[(size_t)(t0 + lane) * Hv + vh];
         bg_in = bg[(size_t)(t0 + lane) * Hv + vh];
     }
-    constexpr int NLV = kC * (DV / 4) / NTHR;
-    float4 va[NLV];
     {
         constexpr int NL = kC * (DK / 4) / NTHR;
         float4 a[NL], b[NL];
@@ -118,6 +193,7 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
             *(float4 *)&sK[tt][x] = float4{a[u].x * keep, a[u].y * keep, a[u].z * keep, a[u].w * keep};
             *(float4 *)&sQ[tt][x] = float4{b[u].x * keep, b[u].y * keep, b[u].z * keep, b[u].w * keep};
         }
+    }
     }
     if (wave == 0) {
         float l = lg_in;
@@ -180,11 +256,13 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
             const float4 o = {e.x * sK[j4 + 0][kk], e.y * sK[j4 + 1][kk], e.z * sK[j4 + 2][kk], e.w * sK[j4 + 3][kk]};
             *(float4 *)(Kt + (slot * NK * 4 + tile) * 256 + l * 4) = o;
         }
+        if constexpr (!FUSED) {
 #pragma unroll
-        for (int u = 0; u < NLV; u++) {
-            const int i = tid + u * NTHR, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
-            const float keep = tt < nt ? 1.f : 0.f;
-            *(float4 *)&sQ[tt][x] = float4{va[u].x * keep, va[u].y * keep, va[u].z * keep, va[u].w * keep};
+            for (int u = 0; u < NLV; u++) {
+                const int i = tid + u * NTHR, tt = i / (DV / 4), x = (i % (DV / 4)) * 4;
+                const float keep = tt < nt ? 1.f : 0.f;
+                *(float4 *)&sQ[tt][x] = float4{va[u].x * keep, va[u].y * keep, va[u].z * keep, va[u].w * keep};
+            }
         }
     }
     if (wave < 4) {
@@ -240,7 +318,7 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 bK[s][ct][i] = sK[16 * s + 4 * g + i][16 * (NCT * wave + ct) + m];
-                bV[s][ct][i] = sQ[16 * s + 4 * g + i][16 * (NCT * wave + ct) + m];
+                bV[s][ct][i] = (FUSED ? sV : sQ)[16 * s + 4 * g + i][16 * (NCT * wave + ct) + m];
             }
 #pragma unroll
     for (int tau = 0; tau < 4; tau++) {
@@ -411,10 +489,12 @@ size_t gdn_wy_scratch_elems(int Hv, int dk, int dv, int T) {
     return nblk * Hv * (3 * (size_t)kC * dk + (size_t)kC * dv + (size_t)kC * kC + kC);
 }
 
-// qn, kn [T, Hk, dk]; vv [T, Hv, dv]; lg, bg [T, Hv] (log decay, beta gate); o_raw [T, Hv*dv].
+// o_raw [T, Hv*dv].  The blocks' inputs come from the layer's inputs (`in`; qn .. bg are then unused
+// and may be null) or, when in is null, from qn, kn [T, Hk, dk]; vv [T, Hv, dv]; lg, bg [T, Hv] (log
+// decay, beta gate) as gdn_chunk_pre_kernel leaves them.
 int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const float *qn, const float *kn,
                   const float *vv, const float *lg, const float *bg, float *scratch, float *ssm,
-                  float *o_raw) {
+                  float *o_raw, const WyInputs *in) {
     if (dk != dv || (dk != 64 && dk != 128))
         return fail(MFA_ERR_SHAPE, "gdn blocked form: dk=%d dv=%d not supported", dk, dv);
     const size_t nblk = ((size_t)T + kC - 1) / kC;
@@ -426,17 +506,20 @@ int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const fl
     float *Ut = Kt + slots * kC * dk;
     float *Mt = Ut + slots * kC * dv;
     float *eLc = Mt + slots * kC * kC;
+    const WyInputs none{};
+#define MFA_WY(DKK, FU)                                                                                             \
+    hipLaunchKernelGGL((gdn_wy_kernel<DKK, FU>), dim3(Hv, (unsigned)nblk), dim3(DKK * 4), 0, s, Hk, Hv, T, qn, kn, vv, \
+                       lg, bg, Wt, Qt, Ut, Mt, Kt, eLc, in ? *in : none)
     if (dk == 128) {
-        hipLaunchKernelGGL((gdn_wy_kernel<128>), dim3(Hv, (unsigned)nblk), dim3(512), 0, s, Hk, Hv, T, qn, kn, vv,
-                           lg, bg, Wt, Qt, Ut, Mt, Kt, eLc);
+        if (in) MFA_WY(128, true); else MFA_WY(128, false);
         hipLaunchKernelGGL((gdn_wy_recur_kernel<128>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, Wt, Qt, Ut,
                            Mt, Kt, eLc, ssm, o_raw);
     } else {
-        hipLaunchKernelGGL((gdn_wy_kernel<64>), dim3(Hv, (unsigned)nblk), dim3(256), 0, s, Hk, Hv, T, qn, kn, vv,
-                           lg, bg, Wt, Qt, Ut, Mt, Kt, eLc);
+        if (in) MFA_WY(64, true); else MFA_WY(64, false);
         hipLaunchKernelGGL((gdn_wy_recur_kernel<64>), dim3(Hv, dv / 16), dim3(256), 0, s, Hk, Hv, T, Wt, Qt, Ut,
                            Mt, Kt, eLc, ssm, o_raw);
     }
+#undef MFA_WY
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }

@@ -315,9 +315,19 @@ size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T);
 // gdn_wy.hip: the recurrence of a chunk in blocked form (blocks of 64 tokens) on the matrix
 // cores, from the per-token operands the chunk's first kernel prepares.
 size_t gdn_wy_scratch_elems(int Hv, int dk, int dv, int T);
+// The layer's inputs, for blocks of the blocked form that compute their own operands from them.
+struct WyInputs {
+    const float *qkv;          // [T, C] the chunk's conv inputs
+    const float *ring;         // [K, C] conv history (input number s in slot s % K)
+    const uint16_t *conv_w;    // [C, K] bf16
+    const float *a_log;        // [Hv]
+    const uint16_t *dt_bias;   // [Hv] bf16
+    const float *alpha, *beta; // [T, Hv]
+    int K, step_mod;
+};
 int launch_gdn_wy(hipStream_t s, int Hk, int Hv, int dk, int dv, int T, const float *qn, const float *kn,
                   const float *vv, const float *lg, const float *bg, float *scratch, float *ssm,
-                  float *o_raw);
+                  float *o_raw, const WyInputs *in = nullptr);
 int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps, int T,
                      const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                      const float *qkv_in, const float *z, const float *alpha, const float *beta,
