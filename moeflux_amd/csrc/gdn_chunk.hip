@@ -284,7 +284,7 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
     float *wy = scratch + chunk_common_elems(Hk, Hv, dk, dv, T);
     const int nvb = (Hv * dv + 255) / 256;
     const bool blocked = T >= kWyMinTokens;
-    if (blocked) {
+    if (blocked && K == 4) {
         // the blocks of the blocked form compute conv, norms and gates themselves
         const WyInputs in{qkv_in, conv_ring, w.conv_w, w.a_log, w.dt_bias, alpha, beta, K, (int)(step % K)};
         MFA_TRY(launch_gdn_wy(s, Hk, Hv, dk, dv, T, nullptr, nullptr, nullptr, nullptr, nullptr, wy, ssm, o_raw, &in));
@@ -298,7 +298,9 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
                                Hk, Hv, dv, K, T, (int)(step % K), w.conv_w, w.a_log, w.dt_bias, conv_ring, qkv_in, alpha, beta, qn, kn,
                                vv, gd, bg, kq, lg);
         MFA_HIP(hipGetLastError());
-        if (dk == 128)
+        if (blocked)
+            MFA_TRY(launch_gdn_wy(s, Hk, Hv, dk, dv, T, qn, kn, vv, lg, bg, wy, ssm, o_raw));
+        else if (dk == 128)
             hipLaunchKernelGGL((gdn_chunk_recur_kernel<128, 128>), dim3(Hv, 128 / 16), dim3(256), 0, s, Hk, Hv, T, qn,
                                kn, vv, gd, bg, kq, ssm, o_raw);
         else

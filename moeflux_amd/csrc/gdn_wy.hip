@@ -110,26 +110,51 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
             al_in = in.a_log[vh];
             dt_in = bf16_bits_to_f32(in.dt_bias[vh]);
         }
-        // conv + SiLU (linear_attn.rs:132-154) of channel c over a run of 16 tokens per unit
+        // conv + SiLU (linear_attn.rs:132-154) of channel c over a run of 16 tokens per unit.
+        // First every request of every unit: a run's TT + 3 inputs, oldest first, are rows of the
+        // chunk, or ring slots for inputs from before it.  Every load is unconditional (the address
+        // is selected; rows past the chunk's end re-read its last row and only feed outputs that
+        // are zeroed below), so all of a thread's requests are in flight at once instead of one
+        // memory round trip per input or per unit.
+        // (Conv width 4 only; the launcher sends other widths through the separate first kernel.)
+        float xs[NU][TT + 3];
+        uint2 wbits[NU];
+        const float *blk_rows = in.qkv + (size_t)t0 * C;   // the block's first row: offsets from here fit 32 bits
 #pragma unroll
         for (int u = 0; u < NU; u++) {
             const int unit = tid + u * NTHR, c = unit % NCONV, run = unit / NCONV;
             const int ch = c < DK ? kh * DK + c : c < 2 * DK ? Hk * DK + kh * DK + (c - DK) : 2 * Hk * DK + vh * DV + (c - 2 * DK);
+            wbits[u] = *(const uint2 *)(in.conv_w + (unsigned)ch * 4u);
+#pragma unroll
+            for (int j = 0; j < TT + 3; j++) {
+                const int rel = TT * run - 3 + j;          // row relative to the block's first
+                const int idx = t0 + rel;
+                const int last = T - 1 - t0;
+                if (rel < 0) {                              // compile-time for all but the first run
+                    const int off = (idx < 0 ? ((in.step_mod + idx + 4) & 3) : rel) * C + ch;
+                    xs[u][j] = (idx < 0 ? in.ring : blk_rows)[off];
+                } else {
+                    xs[u][j] = blk_rows[(rel > last ? last : rel) * C + ch];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NU; u++) {
+            const int unit = tid + u * NTHR, c = unit % NCONV, run = unit / NCONV;
             const int tr = t0 + TT * run;
             int ntr = T - tr;
             ntr = ntr < 0 ? 0 : ntr > TT ? TT : ntr;
-            float o[TT];
-            if (in.K == 4) {
-                conv_silu_run<TT, 4>(in.ring, in.qkv, in.conv_w, C, in.step_mod, tr, ntr, ch, o);
-            } else {
-#pragma unroll
-                for (int i = 0; i < TT; i++)
-                    o[i] = i < ntr ? conv_silu(in.ring, in.qkv, in.conv_w, C, in.K, in.step_mod, tr + i, ch) : 0.f;
-            }
+            const float wt[4] = {bf16_bits_to_f32((uint16_t)(wbits[u].x & 0xffffu)), bf16_bits_to_f32((uint16_t)(wbits[u].x >> 16)),
+                                 bf16_bits_to_f32((uint16_t)(wbits[u].y & 0xffffu)), bf16_bits_to_f32((uint16_t)(wbits[u].y >> 16))};
             float(*dst)[LDK] = c < DK ? sQ : c < 2 * DK ? sK : sV;
             const int cc = c < DK ? c : c < 2 * DK ? c - DK : c - 2 * DK;
 #pragma unroll
-            for (int i = 0; i < TT; i++) dst[TT * run + i][cc] = o[i];
+            for (int i = 0; i < TT; i++) {
+                float acc = 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; k++) acc = fmaf(xs[u][i + k], wt[k], acc);
+                dst[TT * run + i][cc] = i < ntr ? silu_f(acc) : 0.f;
+            }
         }
         if (wave == 0 && lane < nt) {
             // shaders.metal:1321-1326; the decay enters as its logarithm
