@@ -519,8 +519,10 @@ struct MergeExtra {
     int new_bf16;
 };
 
-// The same merge as a launch of its own.
+// The same merge as a launch of its own.  TOK: the launch takes a decode step's new token as
+// one more split (MergeExtra); without it none of that code is compiled in.
 // grid (n_tok * Hq, D/64), 256 threads: one 64-output unit per workgroup.
+template <bool TOK>
 __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int Hq, int nhg, int D, const float *__restrict__ gate, float *__restrict__ out, MergeExtra ex) {
@@ -529,16 +531,20 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const int h = blockIdx.x % Hq, tok = blockIdx.x / Hq;
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const MergeOut mo{gate, out, hpk, Hq, 1, D, ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
-    const int c = blockIdx.y * 64 + (threadIdx.x & 63);
-    merge_span<1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate, out,
-                  threadIdx.x, acc4, ex.gate_stride, mo.token_score(kvh, hg, n),
-                  ex.new_score ? mo.token_value(kvh, c) : 0.f);
+    if constexpr (TOK) {
+        const MergeOut mo{gate, out, hpk, Hq, 1, D, ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
+        const int c = blockIdx.y * 64 + (threadIdx.x & 63);
+        merge_span<1, true>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate,
+                            out, threadIdx.x, acc4, ex.gate_stride, mo.token_score(kvh, hg, n), mo.token_value(kvh, c));
+    } else {
+        merge_span<1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate, out,
+                      threadIdx.x, acc4, D);
+    }
 }
 
 // Few splits (at most NS = 8 or 16, what a launch over many layers or row groups ends up
 // with): one wave per 64 outputs of a (token, head) row, four such units per workgroup.
-template <int NS>
+template <int NS, bool TOK>
 __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const float *__restrict__ part_o, const float *__restrict__ part_ml, int nsplit, int hpk,
     int Hq, int nhg, int D, int n_units, const float *__restrict__ gate, float *__restrict__ out, MergeExtra ex) {
@@ -551,8 +557,9 @@ __global__ __launch_bounds__(256) void sdpa_merge_few_kernel(
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
     const int u = n * per_row + by;   // the unit's index inside its row group
     const MergeOut mo{gate, out, hpk, Hq, (int)(((int64_t)n_units / per_row) / Hq), D,
-                      ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
-    merge_few_units<NS, 1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, kvh, hg, u, u + 1, mo, lane);
+                      TOK ? ex.gate_stride : D, TOK ? ex.new_score : nullptr, TOK ? ex.new_v : nullptr,
+                      TOK ? ex.new_bf16 : 0, nhg};
+    merge_few_units<NS, 1, TOK>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, kvh, hg, u, u + 1, mo, lane);
 }
 
 static void launch_merge_kernels(hipStream_t stream, const float *part_o, const float *part_ml, int splits, int hpk,
@@ -561,15 +568,20 @@ static void launch_merge_kernels(hipStream_t stream, const float *part_o, const 
     const MergeExtra ex = extra ? *extra : MergeExtra{D, nullptr, nullptr, 0};
     const int n_units = n_tok * Hq * (D / 64);
     const dim3 few((n_units + 3) / 4);
-    if (splits <= 8)
-        hipLaunchKernelGGL((sdpa_merge_few_kernel<8>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
-                           n_units, gate, out, ex);
-    else if (splits <= 16)
-        hipLaunchKernelGGL((sdpa_merge_few_kernel<16>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, Hq, nhg, D,
-                           n_units, gate, out, ex);
-    else
-        hipLaunchKernelGGL(sdpa_merge_kernel, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, part_o, part_ml, splits, hpk,
-                           Hq, nhg, D, gate, out, ex);
+#define MFA_MERGE(TOKK)                                                                                                 \
+    do {                                                                                                                \
+        if (splits <= 8)                                                                                                \
+            hipLaunchKernelGGL((sdpa_merge_few_kernel<8, TOKK>), few, dim3(256), 0, stream, part_o, part_ml, splits, hpk, \
+                               Hq, nhg, D, n_units, gate, out, ex);                                                     \
+        else if (splits <= 16)                                                                                          \
+            hipLaunchKernelGGL((sdpa_merge_few_kernel<16, TOKK>), few, dim3(256), 0, stream, part_o, part_ml, splits,   \
+                               hpk, Hq, nhg, D, n_units, gate, out, ex);                                                \
+        else                                                                                                            \
+            hipLaunchKernelGGL(sdpa_merge_kernel<TOKK>, dim3(n_tok * Hq, D / 64), dim3(256), 0, stream, part_o, part_ml, \
+                               splits, hpk, Hq, nhg, D, gate, out, ex);                                                 \
+    } while (0)
+    if (extra) MFA_MERGE(true); else MFA_MERGE(false);
+#undef MFA_MERGE
 }
 
 int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, int hpk, int Hq, int nhg, int D,

@@ -52,7 +52,7 @@ static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 // another wave until the 16 row sums meet in LDS, and every request - split statistics, rows,
 // gate - is made before the first value is used: one memory round trip and one barrier.
 // Called by whole workgroups with a uniform `active` per team; contains two workgroup barriers.
-template <int NU, typename Reader>
+template <int NU, bool TOK = false, typename Reader>
 __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool active, int n, int c0, int64_t orow,
                                   const float *gate, float *out, int ttid, float4 (*acc4)[16][16],
                                   int gate_stride, float tok_score = -__builtin_huge_valf(), float tok_value = 0.f) {
@@ -84,14 +84,15 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
     if (active)
         for (int s = lane + 256; s < nsplit; s += 64) m = fmaxf(m, rd.stat(s * 32 + n));
-    const float M = fmaxf(wave_max(m), tok_score);
+    const float M = TOK ? fmaxf(wave_max(m), tok_score) : wave_max(m);
     auto weight = [&](float ms_) { return (ms_ == neg_inf()) ? 0.f : fast_exp2(ms_ - M); };
     float den = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; r++) den += weight(ms[r]) * ls[r];
     if (active)
         for (int s = lane + 256; s < nsplit; s += 64) den += weight(rd.stat(s * 32 + n)) * rd.stat(s * 32 + n + 16);
-    den = group_sum<64>(den) + weight(tok_score);   // the single position's sum is 1
+    den = group_sum<64>(den);
+    if (TOK) den += weight(tok_score);   // the single position's sum is 1
 
     float4 acc[NU];
 #pragma unroll
@@ -127,7 +128,7 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
         float sum = 0.f;
 #pragma unroll
         for (int x = 0; x < 16; x++) sum += ((const float *)&acc4[u][x][ql])[qc];
-        sum += weight(tok_score) * tok_value;
+        if (TOK) sum += weight(tok_score) * tok_value;
         out[orow * D + c0 + ttid] = (sum / den) * merge_gate(gate, gt_in);
     }
     __syncthreads();   // acc4 may be written again by the next call
@@ -137,7 +138,7 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
 // group: row u / (D/64), channels 64 (u % (D/64)) ...): lane = channel, lane s also holds split
 // s's (max, sum); a lane's output is the weighted sum of one float per split, all of them - for
 // all the wave's units - requested before the first use.  No LDS, no barrier.
-template <int NS, int UPW, typename Reader>
+template <int NS, int UPW, bool TOK = false, typename Reader>
 __device__ inline void merge_few_units(const Reader &rd, int nsplit, int kvh, int hg, int u_first, int u_end,
                                        const MergeOut &mo, int lane) {
     const int D = mo.D, per_row = D / 64;
@@ -157,15 +158,15 @@ __device__ inline void merge_few_units(const Reader &rd, int nsplit, int kvh, in
 #pragma unroll
         for (int s = 0; s < NS; s++) rows[i][s] = rd.row1(((s < nsplit ? s : nsplit - 1) * 16 + n) * D + ch[i]);
         gt_in[i] = (mo.gate && orow[i] >= 0) ? mo.gate[orow[i] * mo.gate_stride + ch[i]] : 0.f;
-        ts_in[i] = mo.token_score(kvh, hg, n);
-        tv_in[i] = mo.new_score ? mo.token_value(kvh, ch[i]) : 0.f;
+        ts_in[i] = TOK ? mo.token_score(kvh, hg, n) : neg_inf();
+        tv_in[i] = TOK ? mo.token_value(kvh, ch[i]) : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < UPW; i++) {
         const float ms = lane < nsplit ? m_in[i] : neg_inf();
-        const float M = fmaxf(wave_max(ms), ts_in[i]);
+        const float M = TOK ? fmaxf(wave_max(ms), ts_in[i]) : wave_max(ms);
         const float w = (ms == neg_inf()) ? 0.f : fast_exp2(ms - M);
-        const float wt = (ts_in[i] == neg_inf()) ? 0.f : fast_exp2(ts_in[i] - M);
+        const float wt = (!TOK || ts_in[i] == neg_inf()) ? 0.f : fast_exp2(ts_in[i] - M);
         const float den = group_sum<64>(w * (lane < nsplit ? l_in[i] : 0.f)) + wt;
         float acc = wt * tv_in[i];
 #pragma unroll
