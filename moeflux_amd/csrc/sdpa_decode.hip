@@ -532,10 +532,10 @@ __global__ __launch_bounds__(256) void sdpa_merge_kernel(
     const int kvh = h / hpk, rr = tok * hpk + h % hpk, hg = rr / 16, n = rr % 16;
     const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
     if constexpr (TOK) {
-        const MergeOut mo{gate, out, hpk, Hq, 1, D, ex.gate_stride, ex.new_score, ex.new_v, ex.new_bf16, nhg};
         const int c = blockIdx.y * 64 + (threadIdx.x & 63);
         merge_span<1, true>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate,
-                            out, threadIdx.x, acc4, ex.gate_stride, mo.token_score(kvh, hg, n), mo.token_value(kvh, c));
+                            out, threadIdx.x, acc4, ex.gate_stride, ex.new_score + ((size_t)kvh * nhg + hg) * 16 + n,
+                            ex.new_v + (size_t)kvh * D + c, ex.new_bf16);
     } else {
         merge_span<1>(PartialsPlain(part_o, part_ml, pid0, D), nsplit, D, true, n, blockIdx.y * 64, blockIdx.x, gate, out,
                       threadIdx.x, acc4, D);

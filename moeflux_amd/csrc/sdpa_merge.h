@@ -27,9 +27,8 @@ struct MergeOut {
     // projected; rounded here as the cache holds it).  Null: none.
     const float *new_score, *new_v;
     int new_bf16, nhg;
-    __device__ float token_score(int kvh, int hg, int n) const {
-        return new_score ? new_score[((size_t)kvh * nhg + hg) * 16 + n] : -__builtin_huge_valf();
-    }
+    // (callers are the TOK instantiations, where both pointers are set: no branch around the loads)
+    __device__ float token_score(int kvh, int hg, int n) const { return new_score[((size_t)kvh * nhg + hg) * 16 + n]; }
     __device__ float token_value(int kvh, int c) const {
         const float v = new_v[(size_t)kvh * D + c];
         return new_bf16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : v;
@@ -55,7 +54,8 @@ static constexpr int kMergeRows = 8;  // partial rows a thread keeps in flight
 template <int NU, bool TOK = false, typename Reader>
 __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool active, int n, int c0, int64_t orow,
                                   const float *gate, float *out, int ttid, float4 (*acc4)[16][16],
-                                  int gate_stride, float tok_score = -__builtin_huge_valf(), float tok_value = 0.f) {
+                                  int gate_stride, const float *tok_score_at = nullptr, const float *tok_value_at = nullptr,
+                                  int tok_bf16 = 0) {
     constexpr int R = kMergeRows / NU;
     const int lane = ttid & 63, dl = ttid & 15, sg = ttid >> 4;
     // split s of row n: maximum at statistic 32 s + n, sum at 32 s + n + 16
@@ -80,6 +80,14 @@ __device__ inline void merge_span(const Reader &rd, int nsplit, int D, bool acti
     }
     const bool writer = active && ttid < 64 * NU;
     const float gt_in = (gate && writer) ? gate[orow * gate_stride + c0 + ttid] : 0.f;
+    // TOK: the row's score against the new token and this thread's element of the token's value row,
+    // requested with everything else (no branch: both addresses are valid for every thread)
+    float tok_score = neg_inf(), tok_value = 0.f;
+    if constexpr (TOK) {
+        tok_score = *tok_score_at;
+        const float v = *tok_value_at;
+        tok_value = tok_bf16 ? bf16_bits_to_f32(f32_to_bf16_bits(v)) : v;
+    }
 
     float m = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
     if (active)
