@@ -42,6 +42,16 @@ __device__ inline float4 lds_f4(const float *p) {
     const gdn_f32x4 v = *reinterpret_cast<const gdn_f32x4 *>(p);
     return float4{v.x, v.y, v.z, v.w};
 }
+// Value head served by the workgroups with x index bx.  Workgroups go to the 8 XCDs in turn, so with a
+// head count that is a multiple of 8 a head's workgroups share an XCD and its L2; heads that share a
+// k head (and read the same q and k inputs) are given x indices 8 apart, the same XCD, so that the
+// second reader of a line finds it in that L2 (block precompute 22.3 -> 21.6 us per 512 tokens).
+__device__ inline int wy_head_of(int bx, int Hk, int Hv) {
+    const int r = Hv / Hk;
+    if (Hv % 8 != 0 || (Hv / 8) % r != 0) return bx;
+    const int x = bx & 7, j = bx >> 3;
+    return (x + 8 * (j / r)) * r + j % r;
+}
 __device__ inline float4 as_f4(wy_f32x4 v) { return float4{v[0], v[1], v[2], v[3]}; }
 // a 16-byte load kept as a vector register value (members of a struct of operands)
 __device__ inline wy_f32x4 load_v4(const float *p) { return *reinterpret_cast<const wy_f32x4 *>(p); }
@@ -85,7 +95,7 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
 
     // heads along x: a head's blocks are produced on the XCD whose L2 the recurrence kernel
     // (heads along x as well) will read them through
-    const int vh = blockIdx.x, blk = blockIdx.y, kh = vh / (Hv / Hk);
+    const int vh = wy_head_of(blockIdx.x, Hk, Hv), blk = blockIdx.y, kh = vh / (Hv / Hk);
     const int t0 = blk * kC;
     const int nt = (T - t0 < kC) ? T - t0 : kC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -389,7 +399,7 @@ __global__ __launch_bounds__(256) void gdn_wy_recur_kernel(
     __shared__ wy_f32x4 s_d[4][64];    // D tiles of the block, by token tile
     __shared__ wy_f32x4 s_st[NK][64];  // the updated state
 
-    const int vh = blockIdx.x, row0 = blockIdx.y * 16;
+    const int vh = wy_head_of(blockIdx.x, Hk, Hv), row0 = blockIdx.y * 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = lane & 15, g = lane >> 4;
     float *srow = ssm + ((size_t)vh * DV + row0 + m) * DK + 4 * g;
