@@ -569,6 +569,25 @@ def bench_snapshot(seed):
             raise RuntimeError(ffi.last_error())
         lib.mfa_sync(ctx.h)
         times["load"].append(time.perf_counter() - t0)
+    # the same through a page-locked buffer of the library's (mfa_host_alloc)
+    pin = lib.mfa_host_alloc(size)
+    if not pin:
+        raise RuntimeError(ffi.last_error())
+    times["save_pinned"], times["load_pinned"] = [], []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        nbytes = lib.mfa_state_save(ctx.h, pin, size)
+        times["save_pinned"].append(time.perf_counter() - t0)
+        if nbytes != size:
+            raise RuntimeError("mfa_state_save: %d of %d bytes" % (nbytes, size))
+        t0 = time.perf_counter()
+        if lib.mfa_state_load(ctx.h, pin, size) != 0:
+            raise RuntimeError(ffi.last_error())
+        lib.mfa_sync(ctx.h)
+        times["load_pinned"].append(time.perf_counter() - t0)
+    if C.string_at(pin, size) != buf.tobytes():
+        raise RuntimeError("snapshot through the page-locked buffer differs")
+    lib.mfa_host_free(pin)
     # the same state as a checkpoint kept on the device (mfa_checkpoint_pos / mfa_restore_to)
     times["checkpoint"], times["restore"] = [], []
     for _ in range(3):
@@ -584,6 +603,9 @@ def bench_snapshot(seed):
     return {"layers": NL, "kv_len": L, "bytes": size, "save_ms": min(times["save"]) * 1e3,
             "load_ms": min(times["load"]) * 1e3, "save_gbps": size / min(times["save"]) / 1e9,
             "load_gbps": size / min(times["load"]) / 1e9,
+            "save_pinned_ms": min(times["save_pinned"]) * 1e3, "load_pinned_ms": min(times["load_pinned"]) * 1e3,
+            "save_pinned_gbps": size / min(times["save_pinned"]) / 1e9,
+            "load_pinned_gbps": size / min(times["load_pinned"]) / 1e9,
             "device_checkpoint_ms": min(times["checkpoint"]) * 1e3,
             "device_restore_ms": min(times["restore"]) * 1e3}
 

@@ -361,6 +361,12 @@ int mfa_linear_state_import(mfa_ctx *ctx, int32_t layer, const float *conv_state
  * byte count or a negative code; mfa_state_load checks the whole buffer before
  * it restores anything (MFA_ERR_STATE for magic, version, shape, truncation,
  * negative length; MFA_ERR_OVERFLOW for a length beyond kv_capacity). */
+/* Page-locked host memory for buffers that cross PCIe whole: a snapshot saved into or loaded
+ * from such a buffer moves at the link's rate, one from malloc'd memory at the rate of the
+ * runtime's staging copies (about a third).  No counterpart in the reference, whose state lives
+ * in host memory.  NULL on failure; mfa_host_free(NULL) is a no-op. */
+void *mfa_host_alloc(int64_t bytes);
+void mfa_host_free(void *p);
 int64_t mfa_state_size(mfa_ctx *ctx);
 int64_t mfa_state_save(mfa_ctx *ctx, uint8_t *buf, int64_t buf_len);
 int mfa_state_load(mfa_ctx *ctx, const uint8_t *buf, int64_t buf_len);

@@ -438,6 +438,31 @@ static int sdpa_stateless(int kv_dtype, int32_t kv_len, int32_t Hq, int32_t Hkv,
     return dout.download(out, qd * 4);
 }
 
+// Device-to-device halves of the export and import calls, enqueued on the context's stream without
+// a synchronisation, for callers that move the state of many layers at once (the snapshot).
+// k_dev, v_dev: [len, num_kv_heads * head_dim] f32; conv_dev: [(K-1) * C] f32, oldest input first.
+int kv_export_to(Ctx *c, FullLayer *f, float *k_dev, float *v_dev) {
+    if (f->len == 0) return MFA_OK;
+    return launch_kv_gather(c->stream, c->cfg.kv_dtype, c->cfg.num_kv_heads, c->cfg.head_dim, c->plane_elems,
+                            f->len, f->k, f->v, k_dev, v_dev);
+}
+int kv_import_from(Ctx *c, FullLayer *f, int32_t len, const float *k_dev, const float *v_dev) {
+    MFA_TRY(truncate_full(c, *f, 0));
+    if (len > 0)
+        MFA_TRY(launch_kv_scatter(c->stream, c->cfg.kv_dtype, 0, c->cfg.num_kv_heads, c->cfg.head_dim,
+                                  c->plane_elems, 0, len, k_dev, v_dev, f->k, f->v));
+    f->len = len;
+    return MFA_OK;
+}
+int linear_export_to(Ctx *c, LinearLayer *l, float *conv_dev) {
+    return launch_conv_ring_export(c->stream, c->conv_dim(), c->cfg.conv_kernel_size, l->step, l->conv_ring, conv_dev);
+}
+int linear_import_from(Ctx *c, LinearLayer *l, const float *conv_dev) {
+    MFA_TRY(launch_conv_ring_import(c->stream, c->conv_dim(), c->cfg.conv_kernel_size, conv_dev, l->conv_ring));
+    l->step = 0;
+    return MFA_OK;
+}
+
 }  // namespace mfa
 
 using namespace mfa;
@@ -1073,6 +1098,25 @@ int mfa_kv_export(mfa_ctx *ctx, int32_t layer, int32_t max_rows, float *k_out, f
                              c->plane_elems, f->len, f->k, f->v, c->stage, c->stage + n));
     MFA_HIP(hipMemcpyAsync(k_out, c->stage, n * 4, hipMemcpyDeviceToHost, c->stream));
     return d2h_sync(c, v_out, c->stage + n, n * 4);
+}
+
+
+void *mfa_host_alloc(int64_t bytes) {
+    if (bytes <= 0) {
+        (void)fail(MFA_ERR_INVALID, "host allocation of %lld bytes", (long long)bytes);
+        return nullptr;
+    }
+    void *p = nullptr;
+    const hipError_t e = hipHostMalloc(&p, (size_t)bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)fail(MFA_ERR_HIP, "hipHostMalloc(%lld): %s", (long long)bytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    return p;
+}
+
+void mfa_host_free(void *p) {
+    if (p) (void)hipHostFree(p);
 }
 
 static int kv_import(Ctx *c, int32_t layer, int32_t len, const void *k, const void *v, int src_bf16) {

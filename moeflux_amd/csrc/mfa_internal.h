@@ -203,6 +203,11 @@ inline Ctx *as_ctx(mfa_ctx *c) { return reinterpret_cast<Ctx *>(c); }
 int full_layer(Ctx *c, int32_t layer, FullLayer **out);
 int linear_layer(Ctx *c, int32_t layer, LinearLayer **out);
 int ensure_stage(Ctx *c, size_t elems);
+// api.hip: device-to-device halves of the state export and import calls (no synchronisation)
+int kv_export_to(Ctx *c, FullLayer *f, float *k_dev, float *v_dev);
+int kv_import_from(Ctx *c, FullLayer *f, int32_t len, const float *k_dev, const float *v_dev);
+int linear_export_to(Ctx *c, LinearLayer *l, float *conv_dev);
+int linear_import_from(Ctx *c, LinearLayer *l, const float *conv_dev);
 
 // ---- kernel launchers (device pointers, asynchronous on `stream`) ------------
 

@@ -36,6 +36,12 @@ static uint32_t get_u32(const uint8_t *p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
 }
 
+// The device image the state is assembled in (save) or unpacked from (load): per layer one segment of
+// the context's staging buffer, 256-byte aligned, holding K rows then V rows, or the conv state (the
+// recurrent state is copied to and from its own allocation).  Offsets in floats.
+static constexpr size_t kSegAlign = 64;
+static size_t seg_round(size_t elems) { return (elems + kSegAlign - 1) / kSegAlign * kSegAlign; }
+
 }  // namespace mfa
 
 using namespace mfa;
@@ -61,19 +67,50 @@ int64_t mfa_state_save(mfa_ctx *ctx, uint8_t *buf, int64_t buf_len) {
     const uint32_t header[kHeaderV2] = {kMagic, kVersion, (uint32_t)c->cfg.num_layers, (uint32_t)c->cfg.full_attn_interval,
                                         (uint32_t)c->cfg.num_kv_heads, (uint32_t)c->cfg.head_dim,
                                         (uint32_t)conv_bytes(c), (uint32_t)ssm_bytes(c), 0u, 0u};
-    size_t off = 0;
+    // every layer's rows are gathered into the device image first, then the copies follow one
+    // another on the stream, and the host waits once
+    size_t img = 0;
+    for (int i = 0; i < c->cfg.num_layers; i++)
+        img += c->kind[i] == 1 ? seg_round(2 * (size_t)c->full[c->slot[i]].len * c->kv_dim()) : seg_round(conv_bytes(c) / 4);
+    MFA_TRY(ensure_stage(c, img));
+    size_t at = 0;
+    for (int i = 0; i < c->cfg.num_layers; i++) {
+        if (c->kind[i] == 1) {
+            FullLayer *f = &c->full[c->slot[i]];
+            const size_t n = (size_t)f->len * c->kv_dim();
+            MFA_TRY(kv_export_to(c, f, c->stage + at, c->stage + at + n));
+            at += seg_round(2 * n);
+        } else {
+            MFA_TRY(linear_export_to(c, &c->lin[c->slot[i]], c->stage + at));
+            at += seg_round(conv_bytes(c) / 4);
+        }
+    }
+    size_t off = kHeaderV2 * 4;
+    at = 0;
+    for (int i = 0; i < c->cfg.num_layers; i++) {
+        if (c->kind[i] == 1) {
+            const size_t n = (size_t)c->full[c->slot[i]].len * c->kv_dim();
+            off += 4;
+            if (n > 0) MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, 2 * n * 4, hipMemcpyDeviceToHost, c->stream));
+            off += 2 * n * 4;
+            at += seg_round(2 * n);
+        } else {
+            MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, conv_bytes(c), hipMemcpyDeviceToHost, c->stream));
+            MFA_HIP(hipMemcpyAsync(buf + off + conv_bytes(c), c->lin[c->slot[i]].ssm, ssm_bytes(c), hipMemcpyDeviceToHost, c->stream));
+            off += conv_bytes(c) + ssm_bytes(c);
+            at += seg_round(conv_bytes(c) / 4);
+        }
+    }
+    MFA_HIP(hipStreamSynchronize(c->stream));
+    // the words the host knows: header and cache lengths
+    off = 0;
     for (uint32_t w : header) { put_u32(buf + off, w); off += 4; }
     for (int i = 0; i < c->cfg.num_layers; i++) {
         if (c->kind[i] == 1) {
             const int32_t len = c->full[c->slot[i]].len;
             put_u32(buf + off, (uint32_t)len);
-            off += 4;
-            const size_t bytes = (size_t)len * row_bytes(c);
-            if (len > 0)
-                MFA_TRY(mfa_kv_export(ctx, i, len, (float *)(buf + off), (float *)(buf + off + bytes)));
-            off += 2 * bytes;
+            off += 4 + 2 * (size_t)len * row_bytes(c);
         } else {
-            MFA_TRY(mfa_linear_state_export(ctx, i, (float *)(buf + off), (float *)(buf + off + conv_bytes(c))));
             off += conv_bytes(c) + ssm_bytes(c);
         }
     }
@@ -131,19 +168,40 @@ int mfa_state_load(mfa_ctx *ctx, const uint8_t *buf, int64_t buf_len) {
             q += bytes;
         }
     }
-    // restore
-    size_t off = header_bytes;
+    // restore: every layer's bytes go to the device image first (a copy from pageable memory has
+    // left the caller's buffer when the call returns), then the kernels unpack them; one wait
+    size_t img = 0, off = header_bytes;
+    for (int i = 0; i < c->cfg.num_layers; i++) {
+        if (c->kind[i] == 1) {
+            const int32_t len = (int32_t)get_u32(buf + off);
+            off += 4 + 2 * (size_t)len * row_bytes(c);
+            img += seg_round(2 * (size_t)len * c->kv_dim());
+        } else {
+            off += conv_bytes(c) + ssm_bytes(c);
+            img += seg_round(conv_bytes(c) / 4);
+        }
+    }
+    MFA_TRY(ensure_stage(c, img));
+    off = header_bytes;
+    size_t at = 0;
     for (int i = 0; i < c->cfg.num_layers; i++) {
         if (c->kind[i] == 1) {
             const int32_t len = (int32_t)get_u32(buf + off);
             off += 4;
-            const size_t bytes = (size_t)len * row_bytes(c);
-            MFA_TRY(mfa_kv_import(ctx, i, len, (const float *)(buf + off), (const float *)(buf + off + bytes)));
-            off += 2 * bytes;
+            const size_t n = (size_t)len * c->kv_dim();
+            if (n > 0) MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, 2 * n * 4, hipMemcpyHostToDevice, c->stream));
+            MFA_TRY(kv_import_from(c, &c->full[c->slot[i]], len, c->stage + at, c->stage + at + n));
+            off += 2 * n * 4;
+            at += seg_round(2 * n);
         } else {
-            MFA_TRY(mfa_linear_state_import(ctx, i, (const float *)(buf + off), (const float *)(buf + off + conv_bytes(c))));
+            LinearLayer *l = &c->lin[c->slot[i]];
+            MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, conv_bytes(c), hipMemcpyHostToDevice, c->stream));
+            MFA_TRY(linear_import_from(c, l, c->stage + at));
+            MFA_HIP(hipMemcpyAsync(l->ssm, buf + off + conv_bytes(c), ssm_bytes(c), hipMemcpyHostToDevice, c->stream));
             off += conv_bytes(c) + ssm_bytes(c);
+            at += seg_round(conv_bytes(c) / 4);
         }
     }
+    MFA_HIP(hipStreamSynchronize(c->stream));
     return MFA_OK;
 }

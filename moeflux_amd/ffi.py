@@ -44,6 +44,8 @@ SIGNATURES = {
     "mfa_set_partial_only": (C.c_int, [vp, i32]),
     "mfa_set_merge": (C.c_int, [vp, i32, i32]),
     "mfa_set_step_launches": (C.c_int, [vp, i32]),
+    "mfa_host_alloc": (vp, [C.c_int64]),
+    "mfa_host_free": (None, [vp]),
     "mfa_kv_append": (C.c_int, [vp, i32, f32p, f32p]),
     "mfa_kv_append_dev": (C.c_int, [vp, i32, f32p, f32p]),
     "mfa_kv_len": (i32, [vp, i32]),

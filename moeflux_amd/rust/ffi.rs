@@ -111,6 +111,8 @@ extern "C" {
     pub fn mfa_set_partial_only(ctx: *mut mfa_ctx, on: i32) -> c_int;
     pub fn mfa_set_merge(ctx: *mut mfa_ctx, in_launch: i32, helper_polls: i32) -> c_int;
     pub fn mfa_set_step_launches(ctx: *mut mfa_ctx, launches: i32) -> c_int;
+    pub fn mfa_host_alloc(bytes: i64) -> *mut c_void;
+    pub fn mfa_host_free(p: *mut c_void);
     pub fn mfa_set_sweep_per_layer(ctx: *mut mfa_ctx, on: i32) -> c_int;
     pub fn mfa_timer_start(ctx: *mut mfa_ctx) -> c_int;
     pub fn mfa_timer_stop(ctx: *mut mfa_ctx, elapsed_ms: *mut f32) -> c_int;

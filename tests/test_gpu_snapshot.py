@@ -77,6 +77,37 @@ def test_snapshot_layout_and_round_trip(mfa, oracle, bf16):
         assert c2.state_save() == blob
 
 
+def test_snapshot_through_a_page_locked_buffer_and_with_an_empty_cache(mfa, oracle):
+    """mfa_host_alloc gives the buffer the copies run fastest with; the bytes are those of a save
+    into ordinary memory.  One full-attention layer holds no positions: its record is the length
+    word alone, and loading it empties that layer's cache."""
+    import ctypes as C
+    from moeflux_amd import ffi
+    lib = ffi.load()
+    case = GdnCase(3, 2, 4, 64, 64, T=4)
+    cfg = _cfg(True)
+    with mfa.Ctx(cfg) as c:
+        _fill(c, case, oracle, True)
+        c.kv_import(1, np.zeros((0, Hkv * D), np.float32), np.zeros((0, Hkv * D), np.float32))
+        assert c.kv_len(1) == 0 and c.kv_len(3) == 40
+        blob = c.state_save()
+        size = c.state_size()
+        assert size == len(blob)
+        pin = lib.mfa_host_alloc(size)
+        assert pin
+        try:
+            assert lib.mfa_state_save(c.h, pin, size) == size
+            assert C.string_at(pin, size) == blob
+            c.memory_clear()
+            assert lib.mfa_state_load(c.h, pin, size) == 0
+            assert c.kv_len(1) == 0 and c.kv_len(3) == 40
+            assert c.state_save() == blob
+        finally:
+            lib.mfa_host_free(pin)
+        assert lib.mfa_host_alloc(0) is None and lib.mfa_host_alloc(-5) is None
+        lib.mfa_host_free(None)
+
+
 def test_snapshot_rejections_leave_the_context_untouched(mfa, oracle):
     from moeflux_amd import MfaError
     case = GdnCase(3, 2, 4, 64, 64, T=4)
