@@ -491,16 +491,20 @@ def bench_prologue(steps, warmup, seed):
     one launch) and the whole layer step from the raw projections (mfa_full_attn_step_dev) in its
     two forms: two launches (the attention launch norms and rotates its own query heads and
     appends the token, the merge takes the token as one more split) and three (prologue,
-    attention, merge)."""
+    attention, merge).  Every call appends a position; the caches start short of 32768 by the
+    number of calls, so that the three measurements run up to the headline's length and not past
+    it.  One more measurement continues from there: just past a length at which every workgroup
+    has one whole pass, the plan changes to half as many workgroups with two passes each."""
     from moeflux_amd import Config, Ctx, ffi
     from moeflux_amd.hip import DeviceArray
     lib = ffi.load()
     Hq, Hkv, d, L, NL = 32, 2, 256, 32768, 8
-    n = (3 * (REPS * steps + warmup) + 8 + NL - 1) // NL + 1
+    per_run = (REPS * steps + warmup + NL - 1) // NL + 1     # positions a measurement adds to a layer
+    L0 = L - 3 * per_run
     ctx = Ctx(Config(num_layers=NL, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
-                     kv_capacity=L + n, kv_dtype=ffi.KV_BF16))
+                     kv_capacity=L + per_run, kv_dtype=ffi.KV_BF16))
     rng = np.random.default_rng(seed)
-    kv = _bf16_bits(rng.standard_normal((L, Hkv * d), dtype=np.float32))
+    kv = _bf16_bits(rng.standard_normal((L0, Hkv * d), dtype=np.float32))
     w = _bf16_bits(np.ones(d, np.float32))
     for l in range(NL):
         ctx.kv_import(l, kv, kv)
@@ -509,7 +513,7 @@ def bench_prologue(steps, warmup, seed):
     k = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
     v = DeviceArray.from_host(rng.standard_normal(Hkv * d).astype(np.float32))
     q, g, o = (DeviceArray((Hq * d,), np.float32, zero=True) for _ in range(3))
-    pos = [L] * NL
+    pos = [L0] * NL
 
     def pro(i):
         l = i % NL
@@ -523,16 +527,23 @@ def bench_prologue(steps, warmup, seed):
             raise RuntimeError(ffi.last_error())
         pos[l] += 1
 
-    _, pro_ms = _timed(ctx, lib, pro, steps, warmup)
     lib.mfa_set_step_launches(ctx.h, 3)
     _, full3_ms = _timed(ctx, lib, full, steps, warmup)
     lib.mfa_set_step_launches(ctx.h, 2)
     _, full2_ms = _timed(ctx, lib, full, steps, warmup)
+    _, pro_ms = _timed(ctx, lib, pro, steps, warmup)
+    if max(pos) > L:
+        raise RuntimeError("the step measurements ran past %d positions" % L)
+    for l in range(NL):      # on from the headline's length exactly
+        while pos[l] < L:
+            full(l)
+    _, past_ms = _timed(ctx, lib, full, steps, warmup)
     alg = 2 * Hq * d * 4 + 2 * Hkv * d * 4 + 2 * Hq * d * 4 + 2 * Hkv * d * 2
-    res = {"shape": "32 Q / 2 KV heads, head_dim 256, bf16 caches of 32768 positions and growing, 8 layers rotated over",
+    res = {"shape": "32 Q / 2 KV heads, head_dim 256, bf16 caches growing to 32768 positions (from %d), 8 layers rotated over" % L0,
            "prologue_us_per_call": pro_ms * 1e3, "prologue_algorithmic_bytes": alg,
            "full_attn_step_us_per_call": full2_ms * 1e3, "launches_per_full_step": 2,
-           "full_attn_step_three_launches_us_per_call": full3_ms * 1e3}
+           "full_attn_step_three_launches_us_per_call": full3_ms * 1e3,
+           "full_attn_step_past_32768_positions_us_per_call": past_ms * 1e3}
     ctx.close()
     for a in (qp, k, v, q, g, o):
         a.free()

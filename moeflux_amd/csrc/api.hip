@@ -311,7 +311,8 @@ static int ensure_workspace_elems(Ctx *c, size_t need_o, size_t need_ml) {
 static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
     const mfa_config &g = c->cfg;
     const int Hq = g.num_attn_heads * layers, Hkv = g.num_kv_heads * layers;
-    int splits = sdpa_pick_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
+    // decode: room for the most splits any length up to kv_len gets (a shorter cache can be split more)
+    int splits = sdpa_max_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
     if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
     MFA_TRY(ensure_tickets(c, (size_t)Hkv * (((size_t)n_tok * (g.num_attn_heads / g.num_kv_heads) + 15) / 16)));
     return ensure_workspace_elems(c, sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok),

@@ -222,6 +222,7 @@ struct SdpaWorkspace {
 };
 bool sdpa_shape_supported(int kv_dtype, int head_dim);
 // Number of splits the launcher will use (for workspace sizing pass kv_len = capacity).
+int sdpa_max_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t max_len, int num_cus, int forced);
 int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int num_cus, int forced);
 size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok = 1);
 size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok = 1);

@@ -639,6 +639,19 @@ int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int n
     return plan_splits(kv_dtype, Hq, Hkv, D, 1, kv_len, num_cus, forced).splits;
 }
 
+// The most splits a decode launch makes at any cache length up to max_len: the plan's split count
+// is not monotonic in the length (whole passes per workgroup), its target is.
+int sdpa_max_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t max_len, int num_cus, int forced) {
+    if (forced > 0) return forced < kMaxSplits ? forced : kMaxSplits;
+    const int hpk = Hq / Hkv;
+    const int64_t nhg = (hpk + 15) / 16, nblk = (max_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
+    int64_t target = num_cus / ((int64_t)Hkv * nhg);
+    if (target < 1) target = 1;
+    if (D <= 128 && nblk >= 8 * 2 * target) target *= 2;
+    if (target > kMaxSplits) target = kMaxSplits;
+    return (int)(target < nblk ? target : (nblk > 0 ? nblk : 1));
+}
+
 size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok) {
     const int64_t nhg = ((int64_t)n_tok * (Hq / Hkv) + 15) / 16;
     return (size_t)Hkv * nhg * splits * 16 * D;
