@@ -85,6 +85,7 @@ struct StepPrologue {
     int64_t cache_pos;         // where its row goes: the cache length before the call
     float *new_score;          // [kv head][row group][16]: q . k_new in log2 units
     void *k_tiled, *v_tiled;   // the planes, to append to
+    int token_split;           // the split whose workgroup also scores and appends the token
 };
 
 // The query operands of the workgroup's 16 rows from the raw q projection: a group of
@@ -209,7 +210,11 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, hg = blockIdx.y, kvh = blockIdx.z;
     // a decode step's launch has one more workgroup per row group, which only scores and appends the new token
-    const int nsplit = gridDim.x - (STEP ? 1 : 0), nhg = gridDim.y;
+    const int nsplit = gridDim.x, nhg = gridDim.y;
+    // A decode step's launch: the workgroup of one split (the last, which has the fewest positions)
+    // also norms and rotates the token's key, scores it against every query row of the group and
+    // appends its row.  Uniform over the workgroup.
+    const bool with_new = STEP && split == sp.token_split;
 
     const int64_t blk_elems = (int64_t)W::BLK * D;
     const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
@@ -228,10 +233,13 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
         for (int i = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; i < fm.n_zero; i += nwg)
             fm.zero[i] = 0ull;
     }
-    if (STEP && split == nsplit) {
-        // The token's own workgroup: its key normed and rotated, its score against every query
-        // row of the group, and its row appended - off the path of the workgroups that stream
-        // the cache.  It leaves no partial; the merge takes the score and the value row directly.
+    if (with_new && b0 >= b1) {
+        // no positions for this split (an empty cache): its partial weighs nothing, the token is all there is
+        if (wave == 0 && g == 0) {
+            const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, neg_inf()), mlb, n * 4, 0, kThrough);
+            __builtin_amdgcn_raw_buffer_store_b32(0u, mlb, (16 + n) * 4, 0, kThrough);
+        }
         StepQuery<KV, D, WAVES * 64> sq;
         sq.request(sp, rows);
         HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
@@ -304,7 +312,7 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
         load_k_part(b0, 0, NLOAD / 2);
         HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
         __syncthreads();
-        sq.finish(sp, rows, qscale, plane_elems, false, qlds, nhg, s_tab);
+        sq.finish(sp, rows, qscale, plane_elems, with_new, qlds, nhg, s_tab);
         load_k_part(b0, NLOAD / 2, NLOAD);
         load_v(b0, 0, kVEarly);
     } else {
@@ -715,8 +723,8 @@ bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim) {
 
 // One decode token of a full-attention layer from its raw projections in two launches: the
 // split-K launch norms and rotates the query heads itself, attends to the len0 positions the
-// cache holds, and its first workgroups score and append the token; the merge adds the token as
-// one more split.  out: [Hq * D].
+// cache holds, and the workgroup of the last split (the one with the fewest positions) also scores
+// and appends the token; the merge adds the token as one more split.  out: [Hq * D].
 int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int64_t len0, size_t plane_elems,
                      void *k_tiled, void *v_tiled, const float *q_proj, const float *k_in, const float *v_in,
                      const uint16_t *q_norm, const uint16_t *k_norm, const float *inv_freq, int rotary_dim,
@@ -726,9 +734,6 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
         return fail(MFA_ERR_SHAPE, "attention step: shape not supported by the two-launch form");
     if (len0 < 0 || pos < 0) return fail(MFA_ERR_INVALID, "attention step: negative position");
     const int hpk = Hq / Hkv;
-    // the token's workgroups (one per row group and kv head) take CUs of their own
-    const int token_wgs = Hkv * ((hpk + 15) / 16);
-    if (num_cus > 2 * token_wgs) num_cus -= token_wgs;
     SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits);
     while (forced_splits <= 0 && plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, 1) > ws.part_o_elems ||
                                                      sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, 1) > ws.part_ml_elems))
@@ -739,9 +744,9 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     const FusedMerge fm{nullptr, nullptr, 0, 0, nullptr, nullptr};
     const StepPrologue sp{q_proj, k_in, v_in, q_norm, k_norm, inv_freq, rotary_dim, eps, pos, len0, new_score,
-                          k_tiled, v_tiled};
+                          k_tiled, v_tiled, plan.splits - 1};
     // rows see positions [0, len0): one token whose own position is not in the cache yet
-    launch_partial_any<true>(kv_dtype, D, plan.waves, stream, dim3(plan.splits + 1, plan.nhg, Hkv), k_tiled, v_tiled,
+    launch_partial_any<true>(kv_dtype, D, plan.waves, stream, dim3(plan.splits, plan.nhg, Hkv), k_tiled, v_tiled,
                              plane_elems, nullptr, hpk, Hq, 1, len0 - 1, (int)plan.bps, qscale, ws.part_o, ws.part_ml,
                              fm, sp);
     MFA_HIP(hipGetLastError());
