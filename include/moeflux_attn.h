@@ -468,6 +468,12 @@ int64_t mfa_debug_kv_offset(int32_t kv_dtype, int32_t is_v, int64_t pos, int32_t
 int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t num_attn_heads, int32_t num_kv_heads,
                              int32_t head_dim, int64_t kv_len, int32_t num_cus,
                              int32_t forced_splits);
+/* The most partitions it uses at any cache length from 1 to max_len, which is what a context's
+ * split-K workspace is sized for: the count is not monotonic in the length (every workgroup
+ * gets whole passes), so the count at the capacity is not the bound. */
+int32_t mfa_debug_max_splits(int32_t kv_dtype, int32_t num_attn_heads, int32_t num_kv_heads,
+                             int32_t head_dim, int64_t max_len, int32_t num_cus,
+                             int32_t forced_splits);
 
 /* A plain device-to-device copy kernel on the context's stream (nbytes read, nbytes
  * written, nbytes a multiple of 16): a launch of known memory traffic, used to scale

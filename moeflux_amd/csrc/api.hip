@@ -1203,6 +1203,14 @@ int32_t mfa_debug_num_splits(int32_t kv_dtype, int32_t Hq, int32_t Hkv, int32_t 
     return sdpa_pick_splits(kv_dtype, Hq, Hkv, D, kv_len, num_cus, forced_splits);
 }
 
+int32_t mfa_debug_max_splits(int32_t kv_dtype, int32_t Hq, int32_t Hkv, int32_t D, int64_t max_len,
+                             int32_t num_cus, int32_t forced_splits) {
+    if (!sdpa_shape_supported(kv_dtype, D) || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || max_len <= 0 ||
+        num_cus <= 0)
+        return -1;
+    return sdpa_max_splits(kv_dtype, Hq, Hkv, D, max_len, num_cus, forced_splits);
+}
+
 int mfa_debug_copy_dev(mfa_ctx *ctx, void *dst_dev, const void *src_dev, size_t nbytes) {
     Ctx *c = as_ctx(ctx);
     if (!c || !dst_dev || !src_dev) return fail(MFA_ERR_INVALID, "NULL argument");

@@ -109,6 +109,7 @@ SIGNATURES = {
     "mfa_gated_rms_norm": (C.c_int, [i32, i32, f32, f32p, f32p, u16p, f32p]),
     "mfa_debug_kv_offset": (C.c_int64, [i32, i32, C.c_int64, i32, i32]),
     "mfa_debug_num_splits": (i32, [i32, i32, i32, i32, C.c_int64, i32, i32]),
+    "mfa_debug_max_splits": (i32, [i32, i32, i32, i32, C.c_int64, i32, i32]),
     "mfa_debug_copy_dev": (C.c_int, [vp, vp, vp, C.c_size_t]),
     "mfa_debug_read_dev": (C.c_int, [vp, vp, C.c_size_t, C.c_int32]),
     "mfa_debug_fill_workspace": (C.c_int, [vp, C.c_uint32]),

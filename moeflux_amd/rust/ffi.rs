@@ -152,6 +152,8 @@ extern "C" {
     pub fn mfa_debug_kv_offset(kv_dtype: i32, is_v: i32, pos: i64, x: i32, head_dim: i32) -> i64;
     pub fn mfa_debug_num_splits(kv_dtype: i32, num_attn_heads: i32, num_kv_heads: i32, head_dim: i32,
         kv_len: i64, num_cus: i32, forced_splits: i32) -> i32;
+    pub fn mfa_debug_max_splits(kv_dtype: i32, num_attn_heads: i32, num_kv_heads: i32, head_dim: i32,
+        max_len: i64, num_cus: i32, forced_splits: i32) -> i32;
     pub fn mfa_debug_copy_dev(ctx: *mut mfa_ctx, dst_dev: *mut c_void, src_dev: *const c_void,
         nbytes: usize) -> c_int;
     pub fn mfa_debug_read_dev(ctx: *mut mfa_ctx, src_dev: *const c_void, nbytes: usize, workgroups: i32) -> c_int;

@@ -56,6 +56,30 @@ def test_tiling_rejects_bad_arguments():
     assert lib.mfa_debug_kv_offset(9, 0, 0, 0, 256) == -1
 
 
+def test_workspace_bound_covers_every_length_up_to_the_capacity():
+    """The split count falls and rises with the length (1024 blocks: 128 splits of one pass; 1025
+    blocks: 65 splits of two), so a context sizes its split-K workspace by a bound over all lengths
+    up to its capacity, not by the count at the capacity."""
+    lib = ffi.load()
+    ns, mx = lib.mfa_debug_num_splits, lib.mfa_debug_max_splits
+    assert ns(ffi.KV_BF16, 32, 2, 256, 32768, 256, 0) == 128
+    assert ns(ffi.KV_BF16, 32, 2, 256, 32800, 256, 0) == 65
+    assert mx(ffi.KV_BF16, 32, 2, 256, 32800, 256, 0) >= 128
+    rng = np.random.default_rng(5)
+    shapes = [(ffi.KV_BF16, 32, 2, 256), (ffi.KV_F32, 32, 4, 128), (ffi.KV_BF16, 64, 2, 128), (ffi.KV_BF16, 8, 8, 64),
+              (ffi.KV_F32, 40, 2, 256), (ffi.KV_BF16, 32 * 12, 2 * 12, 256)]
+    for kv, Hq, Hkv, d in shapes:
+        for cap in (1, 100, 4096, 8191, 32800, 65536, 131072):
+            for forced in (0, 3, 129, 300):
+                bound = mx(kv, Hq, Hkv, d, cap, 256, forced)
+                assert bound >= 1
+                lens = {1, cap, max(1, cap - 1), max(1, cap // 2)} | {int(x) for x in rng.integers(1, cap + 1, 40)}
+                for L in sorted(lens):
+                    got = ns(kv, Hq, Hkv, d, L, 256, forced)
+                    assert 1 <= got <= bound, (kv, Hq, Hkv, d, cap, forced, L, got, bound)
+    assert mx(ffi.KV_BF16, 30, 4, 128, 64, 256, 0) == -1
+
+
 def test_split_partitioning():
     lib = ffi.load()
     ns = lib.mfa_debug_num_splits
