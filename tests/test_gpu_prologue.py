@@ -198,6 +198,35 @@ def test_two_launch_step_equals_three_launch_step(mfa, oracle, bf16, Hq, Hkv, d,
         assert np.array_equal(ka, kb) and np.array_equal(va, vb)
 
 
+@pytest.mark.parametrize("L0", [31, 32, 255, 256, 257, 2047, 2048, 2049, 8191, 8192, 8193])
+def test_two_launch_step_at_the_edges_of_the_split_plan(mfa, oracle, L0):
+    """The token rides in the last split's workgroup: lengths at which that split is full, holds one
+    block, or holds a single position, either side of the lengths at which the plan changes."""
+    Hq, Hkv, d, steps = 32, 2, 256, 2
+    rng, qn, kn = _case(7 * L0 + 1, Hq, Hkv, d)
+    k0 = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal((L0, Hkv * d)).astype(np.float32)))
+    v0 = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal((L0, Hkv * d)).astype(np.float32)))
+    kc = np.concatenate([k0, np.zeros((steps, Hkv * d), np.float32)])
+    vc = np.concatenate([v0, np.zeros((steps, Hkv * d), np.float32)])
+    with _ctx(mfa, Hq, Hkv, d, L0 + steps, bf16=True) as a, _ctx(mfa, Hq, Hkv, d, L0 + steps, bf16=True) as b:
+        b.set_step_launches(3)
+        for c in (a, b):
+            c.set_full_weights(0, qn, kn)
+            c.kv_import(0, k0, v0)
+        for t in range(steps):
+            pos = L0 + t
+            qp = rng.standard_normal(Hq * 2 * d).astype(np.float32)
+            k, v = rng.standard_normal(Hkv * d).astype(np.float32), rng.standard_normal(Hkv * d).astype(np.float32)
+            o2, o3 = a.full_attn_step(0, pos, qp, k, v), b.full_attn_step(0, pos, qp, k, v)
+            rq, rg, rk, rv = oracle.attn_prologue(pos, Hq, Hkv, d, d // 4, THETA, 1e-6, qn, kn, qp, k, v)
+            kc[pos], vc[pos] = (oracle.bf16_to_f32(oracle.f32_to_bf16(x)) for x in (rk, rv))
+            ref = oracle.sdpa(pos + 1, Hq, Hkv, d, rq, rg, kc[:pos + 1], vc[:pos + 1])
+            assert rel_err(o2, o3) <= 1e-4, (t, rel_err(o2, o3))
+            assert rel_err(o2, ref) <= 2e-3, (t, rel_err(o2, ref))
+        (ka, va), (kb, vb) = a.kv_export(0), b.kv_export(0)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+
+
 def test_two_launch_step_with_forced_splits_and_errors(mfa, oracle):
     """The split count does not change the two-launch step's result beyond rounding, a full cache
     is refused before anything is appended, and weights must be set."""
