@@ -31,8 +31,9 @@
 //     parts of the 16 positions followed by their lo parts, so that with P = [p_hi | p_hi]
 //     one instruction adds x_hi p_hi + x_lo p_hi and a second with [p_lo | p_lo] adds x_hi p_lo
 //     (and x_lo p_lo, which comes for free).
-//     The value waves fetch and split 12 of a block's 16 latent rows (two channels per
-//     thread), the score waves the other 4 and the rotary keys, which evens out the two roles.
+//     The value waves fetch and split 6 of a block's 16 latent rows (two channels per
+//     thread), the score waves the other 10 and the rotary keys: the split at which the call is
+//     fastest (12 / 4, which evens out the clocks the two roles spend per block, is 4 % slower).
 //     Partials (unnormalised O, running max and sum per head) go to the workspace in the
 //     layout of the decode kernel's partials, and sdpa_merge_kernel combines them.
 #include "sdpa_wave.h"
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
     static_assert(NROLE == 256 && R == 512 && P == 64, "the staging maps 256 threads per role onto a 16 x (512 + 64) block");
     constexpr int KPLANE = kMlaBlk * KROW * 2;           // bytes of one plane (hi or lo) of a block
     constexpr int KBUF = 2 * KPLANE;                     // one buffer
-    constexpr int VPOS = 12;              // positions of a block whose latent rows the value waves stage; the score waves take the rest
+    constexpr int VPOS = 6;              // positions of a block whose latent rows the value waves stage; the score waves take the rest
     __shared__ __attribute__((aligned(16))) unsigned char smem[3 * KBUF];
     __shared__ __attribute__((aligned(16))) uint16_t pbuf[2][HG][2][16][kMlaBlk];  // weights [buffer][group][hi|lo][head][position]
     __shared__ float abuf[2][HG][16];                                             // rescale factor of a block, per head
