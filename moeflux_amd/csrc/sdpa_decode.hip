@@ -209,7 +209,6 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int split = blockIdx.x, hg = blockIdx.y, kvh = blockIdx.z;
-    // a decode step's launch has one more workgroup per row group, which only scores and appends the new token
     const int nsplit = gridDim.x, nhg = gridDim.y;
     // A decode step's launch: the workgroup of one split (the last, which has the fewest positions)
     // also norms and rotates the token's key, scores it against every query row of the group and
