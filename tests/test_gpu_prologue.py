@@ -227,6 +227,50 @@ def test_two_launch_step_at_the_edges_of_the_split_plan(mfa, oracle, L0):
         assert np.array_equal(ka, kb) and np.array_equal(va, vb)
 
 
+def test_two_launch_step_on_seeded_random_shapes(mfa, oracle):
+    """Head counts, widths, cache kinds, lengths and forced split counts drawn at random (seeded):
+    two launches against three and against the oracle's composition."""
+    rng0 = np.random.default_rng(20240611)
+    for case in range(14):
+        d = int(rng0.choice([64, 128, 256]))
+        Hkv = int(rng0.choice([1, 2, 4]))
+        hpk = int(rng0.choice([1, 4, 8, 16, 20]))
+        Hq = Hkv * hpk
+        bf16 = bool(rng0.integers(0, 2))
+        L0 = int(rng0.choice([0, 1, 15, 16, 17, 100, 513, 1999, 5000]))
+        forced = int(rng0.choice([0, 0, 1, 2, 5, 37]))
+        rng, qn, kn = _case(1000 + case, Hq, Hkv, d)
+        k0 = rng.standard_normal((L0, Hkv * d)).astype(np.float32)
+        v0 = rng.standard_normal((L0, Hkv * d)).astype(np.float32)
+        if bf16:
+            k0, v0 = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k0, v0))
+        kc = np.concatenate([k0, np.zeros((2, Hkv * d), np.float32)])
+        vc = np.concatenate([v0, np.zeros((2, Hkv * d), np.float32)])
+        tag = (case, Hq, Hkv, d, bf16, L0, forced)
+        with _ctx(mfa, Hq, Hkv, d, L0 + 2, bf16=bf16) as a, _ctx(mfa, Hq, Hkv, d, L0 + 2, bf16=bf16) as b:
+            b.set_step_launches(3)
+            for c in (a, b):
+                c.set_full_weights(0, qn, kn)
+                if forced:
+                    c.set_num_splits(forced)
+                if L0:
+                    c.kv_import(0, k0, v0)
+            for t in range(2):
+                pos = L0 + t
+                qp = rng.standard_normal(Hq * 2 * d).astype(np.float32)
+                k, v = rng.standard_normal(Hkv * d).astype(np.float32), rng.standard_normal(Hkv * d).astype(np.float32)
+                o2, o3 = a.full_attn_step(0, pos, qp, k, v), b.full_attn_step(0, pos, qp, k, v)
+                rq, rg, rk, rv = oracle.attn_prologue(pos, Hq, Hkv, d, d // 4, THETA, 1e-6, qn, kn, qp, k, v)
+                if bf16:
+                    rk, rv = (oracle.bf16_to_f32(oracle.f32_to_bf16(x)) for x in (rk, rv))
+                kc[pos], vc[pos] = rk, rv
+                ref = oracle.sdpa(pos + 1, Hq, Hkv, d, rq, rg, kc[:pos + 1], vc[:pos + 1])
+                assert rel_err(o2, o3) <= (1e-4 if bf16 else TOL_F32), (tag, t, rel_err(o2, o3))
+                assert rel_err(o2, ref) <= (2e-3 if bf16 else TOL_F32), (tag, t, rel_err(o2, ref))
+            (ka, va), (kb, vb) = a.kv_export(0), b.kv_export(0)
+            assert np.array_equal(ka, kb) and np.array_equal(va, vb), tag
+
+
 def test_two_launch_step_with_forced_splits_and_errors(mfa, oracle):
     """The split count does not change the two-launch step's result beyond rounding, a full cache
     is refused before anything is appended, and weights must be set."""
