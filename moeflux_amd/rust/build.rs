@@ -14,9 +14,11 @@ fn main() {
     cmd.args(["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-ffp-contract=off"])
         .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"])
         .arg("-I").arg(root.join("include")).arg("-I").arg(&csrc);
+    // every .hip file under csrc/, in sorted order (a test holds this list to the directory)
     for f in [
-        "api.hip", "kv_cache.hip", "sdpa_decode.hip", "sdpa_prefill.hip", "attn_kernels.hip", "gdn.hip",
-        "gdn_chunk.hip", "gdn_wy.hip", "attn_prologue.hip", "snapshot.hip", "dequant_matvec.hip", "mla_sdpa.hip", "checkpoint.hip",
+        "api.hip", "attn_kernels.hip", "attn_prologue.hip", "checkpoint.hip", "dequant_matvec.hip", "gdn.hip",
+        "gdn_chunk.hip", "gdn_wy.hip", "kv_cache.hip", "mla_sdpa.hip", "sdpa_decode.hip", "sdpa_prefill.hip",
+        "sdpa_static.hip", "snapshot.hip",
     ] {
         println!("cargo:rerun-if-changed=csrc/{f}");
         cmd.arg(csrc.join(f));

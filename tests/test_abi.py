@@ -133,3 +133,17 @@ def test_python_mirror_fails_loudly_without_the_library(monkeypatch, tmp_path):
     monkeypatch.setattr(ffi, "_LIB_PATH", str(tmp_path / "missing.so"))
     with pytest.raises(ImportError, match="no CPU fallback"):
         ffi.load()
+
+
+def test_rust_build_script_compiles_every_hip_source():
+    """moeflux_amd/rust/build.rs names its sources one by one; the list is held to csrc/*.hip
+    so that a new source cannot be left out of the library the Rust crate links."""
+    rs = open(os.path.join(ROOT, "moeflux_amd", "rust", "build.rs")).read()
+    body = rs[rs.index("for f in ["):rs.index("] {")]
+    listed = re.findall(r'"([a-z0-9_]+\.hip)"', body)
+    on_disk = sorted(f for f in os.listdir(os.path.join(ROOT, "moeflux_amd", "csrc")) if f.endswith(".hip"))
+    assert listed == on_disk
+    # the flags that change results are the Python build's too
+    from moeflux_amd import build as hip_build
+    for flag in ("--offload-arch=gfx950", "-ffp-contract=off", "-packed-fp32-ops"):
+        assert flag in rs and any(flag in f for f in hip_build.FLAGS), flag
