@@ -758,7 +758,7 @@ def main():
                     help="time launches that only read 64 MiB (the memory system's ceiling at the headline launch size) and exit")
     ap.add_argument("--tokens", type=int, default=512, help="chunk length for --only c4")
     ap.add_argument("--f4-len", type=int, default=0, help="one cache length for --only f4 (default: 4096 and 32768)")
-    ap.add_argument("--only", choices=["c2", "c4", "c5", "f1", "f2", "f3", "f4"], default=None,
+    ap.add_argument("--only", choices=["c1", "c2", "c4", "c5", "f1", "f2", "f3", "f4"], default=None,
                     help="run one secondary configuration alone (for profiling) and print its figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -772,6 +772,10 @@ def main():
         calibrate_read()
         return
 
+    if a.only == "c1":
+        r, _ = bench_sdpa("c1", 32, 4, 128, 4096, False, 24, a.steps, a.warmup, 0xC0FFEE + 1)
+        print(json.dumps({"c1_gqa_decode_f32_L4096": r}))
+        return
     if a.only == "c2":
         print(json.dumps({"c2_gated_deltanet_step": bench_gdn("c2", 16, 32, 128, 128, 160, a.steps, a.warmup, 0xC0FFEE + 2)}))
         return

@@ -10,6 +10,8 @@
 //   O  = diag(e^L) Q S0^T + M D
 //   S' = e^{L_C} S0 + D^T diag(e^{L_C-L}) K
 // are the same d_t, o_t and final state (exact arithmetic; f32 rounding differs at 1e-6).
+// A token whose decay is zero (the reference's exp underflows, or its softplus overflows) starts L
+// afresh: factors across it are exactly 0, as they are token by token.
 // Everything before D depends on the inputs only and is computed for all blocks of the
 // chunk at once (gdn_wy_kernel, one workgroup per (block, value head)); the four
 // products that involve the state run block after block with the state in registers
@@ -92,6 +94,7 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     __shared__ __align__(16) float sA[kC][LDC];
     __shared__ __align__(16) float sT[kC][LDC];
     __shared__ __align__(16) float sL[kC], sB[kC], sCw[kC], sKd[kC];
+    __shared__ int sR[kC];
 
     // heads along x: a head's blocks are produced on the XCD whose L2 the recurrence kernel
     // (heads along x as well) will read them through
@@ -231,18 +234,33 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
     }
     }
     if (wave == 0) {
-        float l = lg_in;
+        // Cumulative log decay, restarted after every token whose decay is zero: where the
+        // reference's exp() underflows (log g below log FLT_MIN; -inf when its softplus overflows,
+        // linear_attn.rs:357-370) the token forgets everything before it, and no factor e^{L_i-L_j}
+        // may be formed across it (-inf - -inf).  sR[t] is the last such token up to and
+        // including t (-1: none); a pair (row, col) decays to exactly 0 when sR[row] > col.
+        const bool dead = lg_in < -87.3f;
+        float l = dead ? 0.f : lg_in;
+        bool seg = dead;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
             const float u = __shfl_up(l, d, 64);
-            if (lane >= d) l += u;
+            const int su = __shfl_up((int)seg, d, 64);
+            if (lane >= d) {
+                if (!seg) l += u;
+                seg = seg || su;
+            }
         }
+        const unsigned long long kills = __ballot(dead) & ((2ull << lane) - 1ull);
+        const int r = kills ? 63 - __builtin_clzll(kills) : -1;
         const float b = bg_in;
+        const float el = r >= 0 ? 0.f : expf(l);      // decay since the block's first token
         sL[lane] = l;
+        sR[lane] = r;
         sB[lane] = b;
-        sCw[lane] = b * expf(l);
-        eLc[slot * kC + lane] = expf(l);
-        sKd[lane] = expf(__shfl(l, 63, 64) - l);  // e^{L_C - L_t}
+        sCw[lane] = b * el;
+        eLc[slot * kC + lane] = el;
+        sKd[lane] = __shfl(r, 63, 64) > lane ? 0.f : expf(__shfl(l, 63, 64) - l);  // e^{L_C - L_t}
     }
     __syncthreads();
 
@@ -266,7 +284,7 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
         for (int i = 0; i < 4; i++) {
             const int row = 16 * I + 4 * g + i;
             const float dl = sL[row] - sL[col];
-            const float d = __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);  // v_exp_f32: 1 ulp
+            const float d = sR[row] > col ? 0.f : __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);  // v_exp_f32: 1 ulp
             if (kind == 0) sA[row][col] = (col < row) ? sB[row] * d * acc[i] : 0.f;
             else  // to tile (I, J) in A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
                 Mt[((slot * 4 + I) * 4 + J) * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = (col <= row) ? d * acc[i] : 0.f;
