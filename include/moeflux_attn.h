@@ -100,18 +100,6 @@ int mfa_set_linear_weights(mfa_ctx *ctx, int32_t layer, const uint16_t *conv_w_b
  * the reference checks tiled against single-shot MLA (tests/mla_sdpa_tiled.rs:
  * 176-216). */
 int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits);
-/* How the split-K partials are combined; no counterpart in the reference, and no result
- * depends on it (tests check exactly that, bit for bit).  By default the merge is a second,
- * small launch behind the attention launch.  in_launch != 0 lets the attention launch merge
- * them itself: every workgroup takes a ticket of its row group once its partial is in memory,
- * the one that draws the last ticket merges the group, and, when a group has many splits,
- * workgroups that finished a moment earlier look on for at most `helper_polls` reads of the
- * group's record (-1 = the default, 0 = nobody waits) and share the work when the last one
- * arrives in time; no workgroup ever depends on another one's progress.  One launch instead
- * of two, for callers that count launches; on MI355X it is the slower of the two (a hop
- * between workgroups through memory - store, ticket, load - measured 2 to 3 us each, against
- * 1.4 us for the boundary between two launches), which is why it is not the default. */
-int mfa_set_merge(mfa_ctx *ctx, int32_t in_launch, int32_t helper_polls);
 /* Measurement aid with no reference counterpart: when `on` is non-zero the
  * decode entry points launch only the split-K partial kernel (no merge, `out`
  * is not written), so that a timed loop isolates the kernel that streams the

@@ -61,24 +61,7 @@ int ensure_stage(Ctx *c, size_t elems) {
 }
 
 static SdpaWorkspace workspace(Ctx *c) {
-    return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems, &c->tickets, c->merge_wait,
-                         c->separate_merge};
-}
-
-// Ticket records for at least `groups` row groups (kv heads x 16-row groups of one launch), zeroed.
-static int ensure_tickets(Ctx *c, size_t groups) {
-    TicketRecords &t = c->tickets;
-    if (groups <= t.cap) return MFA_OK;
-    MFA_HIP(hipStreamSynchronize(c->stream));
-    if (t.dev) MFA_HIP(hipFree(t.dev));
-    t = TicketRecords{};
-    size_t cap = 4096;
-    while (cap < groups) cap *= 2;
-    MFA_HIP(hipMalloc((void **)&t.dev, 2 * cap * sizeof(unsigned long long)));
-    MFA_HIP(hipMemsetAsync(t.dev, 0, 2 * cap * sizeof(unsigned long long), c->stream));
-    MFA_HIP(hipStreamSynchronize(c->stream));
-    t.cap = cap;
-    return MFA_OK;
+    return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems};
 }
 
 static int h2d(Ctx *c, void *dst, const void *src, size_t bytes) {
@@ -100,7 +83,6 @@ static void destroy(Ctx *c) {
         if (p) (void)hipFree(p);
     if (c->part_o) (void)hipFree(c->part_o);
     if (c->part_ml) (void)hipFree(c->part_ml);
-    if (c->tickets.dev) (void)hipFree(c->tickets.dev);
     if (c->stage) (void)hipFree(c->stage);
     if (c->gdn_scratch) (void)hipFree(c->gdn_scratch);
     if (c->qg_chunk) (void)hipFree(c->qg_chunk);
@@ -199,8 +181,7 @@ static int create(const mfa_config *cfg, Ctx **out) {
     c->full.resize(nfull);
     c->lin.resize(nlin);
     if (nfull) {
-        const int blk = cfg->kv_dtype == MFA_KV_BF16 ? 32 : 16;
-        c->cap_pad = ((int64_t)cfg->kv_capacity + blk - 1) / blk * blk;
+        c->cap_pad = ((int64_t)cfg->kv_capacity + kKvChunk - 1) / kKvChunk * kKvChunk;
         c->plane_elems = (size_t)c->cap_pad * cfg->head_dim;
         const size_t bytes = c->plane_elems * cfg->num_kv_heads * c->kv_elem_size();
         // One allocation for all layers' K planes and one for their V planes, layer-major:
@@ -228,14 +209,14 @@ static int create(const mfa_config *cfg, Ctx **out) {
         c->step_score = (float *)sc;
         // variants.rs:245-250, 369: a quarter of the head is rotated, theta = 1e7
         MFA_TRY(set_rope(c, 1.0e7f, cfg->head_dim / 4));
-        int splits = sdpa_pick_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
-                                      cfg->head_dim, cfg->kv_capacity, c->num_cus, 0);
+        // room for the most splits any cache length up to the capacity gets
+        int splits = sdpa_max_splits(cfg->kv_dtype, cfg->num_attn_heads, cfg->num_kv_heads,
+                                     cfg->head_dim, cfg->kv_capacity, c->num_cus, 0);
         if (splits < 128) splits = 128;
         c->part_o_elems = sdpa_workspace_o_elems(cfg->num_attn_heads, cfg->num_kv_heads, cfg->head_dim, splits);
         c->part_ml_elems = sdpa_workspace_ml_elems(cfg->num_attn_heads, cfg->num_kv_heads, splits);
         MFA_HIP(hipMalloc((void **)&c->part_o, c->part_o_elems * sizeof(float)));
         MFA_HIP(hipMalloc((void **)&c->part_ml, c->part_ml_elems * sizeof(float)));
-        MFA_TRY(ensure_tickets(c, 4096));
     }
     if (nlin) {
         const size_t C = (size_t)c->conv_dim(), K = (size_t)cfg->conv_kernel_size;
@@ -314,7 +295,6 @@ static int ensure_workspace(Ctx *c, int n_tok, int64_t kv_len, int layers = 1) {
     // decode: room for the most splits any length up to kv_len gets (a shorter cache can be split more)
     int splits = sdpa_max_splits(g.kv_dtype, Hq, Hkv, g.head_dim, kv_len, c->num_cus, c->forced_splits);
     if (n_tok > 1) splits = 1;  // the launcher splits a chunk less; one split always fits its plan
-    MFA_TRY(ensure_tickets(c, (size_t)Hkv * (((size_t)n_tok * (g.num_attn_heads / g.num_kv_heads) + 15) / 16)));
     return ensure_workspace_elems(c, sdpa_workspace_o_elems(Hq, Hkv, g.head_dim, splits, n_tok),
                                   sdpa_workspace_ml_elems(Hq, Hkv, splits, n_tok));
 }
@@ -402,8 +382,7 @@ static int sdpa_stateless(int kv_dtype, int32_t kv_len, int32_t Hq, int32_t Hkv,
     if (Hq % Hkv != 0) return fail(MFA_ERR_INVALID, "num_attn_heads %d %% num_kv_heads %d != 0", Hq, Hkv);
     if (!sdpa_shape_supported(kv_dtype, D)) return fail(MFA_ERR_SHAPE, "head_dim %d not supported", D);
     const size_t es = kv_dtype == MFA_KV_BF16 ? 2 : 4;
-    const int blk = kv_dtype == MFA_KV_BF16 ? 32 : 16;
-    const int64_t cap = ((int64_t)kv_len + blk - 1) / blk * blk;
+    const int64_t cap = ((int64_t)kv_len + kKvChunk - 1) / kKvChunk * kKvChunk;
     const size_t plane = (size_t)cap * D;
     const size_t qd = (size_t)Hq * D, rows = (size_t)kv_len * Hkv * D;
     int ncu = 256;
@@ -524,16 +503,6 @@ int mfa_set_num_splits(mfa_ctx *ctx, int32_t num_splits) {
     return MFA_OK;
 }
 
-int mfa_set_merge(mfa_ctx *ctx, int32_t in_launch, int32_t helper_polls) {
-    Ctx *c = as_ctx(ctx);
-    if (!c) return fail(MFA_ERR_INVALID, "NULL context");
-    if (helper_polls < -1 || helper_polls > (1 << 20))
-        return fail(MFA_ERR_INVALID, "helper_polls must be -1 (default) or in [0, 2^20] (got %d)", helper_polls);
-    c->separate_merge = in_launch ? 0 : 1;
-    c->merge_wait = helper_polls < 0 ? kDefaultMergeWait : helper_polls;
-    return MFA_OK;
-}
-
 int mfa_set_step_launches(mfa_ctx *ctx, int32_t launches) {
     Ctx *c = as_ctx(ctx);
     if (!c) return fail(MFA_ERR_INVALID, "NULL context");
@@ -651,7 +620,7 @@ static int full_attn_step_dev(Ctx *c, FullLayer *f, int32_t pos, const float *q_
     const mfa_config &g = c->cfg;
     const size_t qd = (size_t)c->q_dim();
     const int32_t len0 = f->len;
-    if (c->step_launches == 2 && !c->partial_only && c->separate_merge &&
+    if (c->step_launches == 2 && !c->partial_only &&
         sdpa_step_supported(g.kv_dtype, g.num_attn_heads, g.num_kv_heads, g.head_dim, c->rotary_dim)) {
         if (!f->norms_set) return fail(MFA_ERR_INVALID, "q/k norm weights not set (mfa_set_full_weights)");
         if (pos < 0) return fail(MFA_ERR_INVALID, "attention prologue: pos %d < 0", pos);

@@ -49,7 +49,7 @@ struct Sizes {
 Sizes sizes_of(const Ctx *c) {
     Sizes s{};
     if (!c->full.empty()) {
-        s.blk = c->cfg.kv_dtype == MFA_KV_BF16 ? 32 : 16;
+        s.blk = kKvChunk;   // K is stored in chunks of 64 positions, which are whole blocks of V
         s.block_bytes = (size_t)s.blk * c->cfg.head_dim * c->kv_elem_size();
         s.plane_bytes = c->plane_elems * c->kv_elem_size();
     }

@@ -49,27 +49,30 @@ __host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
 }
 
 // ---- KV cache tiling ---------------------------------------------------------
-// The device KV cache is stored in the order the decode kernel's MFMA operands
-// consume it, so that every wave-level load is one contiguous 1 KiB run and
-// goes straight from HBM into matrix-core operand registers.
+// The device KV cache is stored in the order the attention kernels' MFMA operands
+// consume it, so that every wave-level load is one contiguous 1 KiB run that goes
+// straight from HBM into matrix-core operand registers, and so that the four waves of a
+// decode workgroup, reading side by side, sweep memory in one contiguous stream.
 //
-// One plane per (layer, K|V, kv head).  Positions are grouped in blocks
-// (32 positions for bf16, 16 for f32); a block of one plane is contiguous.
+// One plane per (layer, K|V, kv head).  K is grouped in chunks of 64 positions (KCH), V in
+// blocks of 32 (bf16) or 16 (f32) positions (BLK); a chunk and a block are contiguous.
 //
-// bf16, block of 32 positions, element (p, x) with p in [0,32), x in [0,D):
-//   K: [step = x/32][sub = p/16][chunk = (x%32)/8][row = p%16][e = x%8]
-//   V: [dt = x/16][g = (p%16)/4][m = x%16][e = 4*(p/16) + p%4]
-// f32, block of 16 positions:
-//   K: [chunk = x/4][row = p][e = x%4]
-//   V: [dt = x/16][g = p/4][m = x%16][j = p%4]
+// K, chunk of 64 positions, element (p, x) with p in [0,64), x in [0,D).  A 1 KiB piece holds
+// 16 positions (sub-tile p/16) of one MFMA k-step; the four sub-tiles of a k-step are adjacent:
+//   bf16: [step = x/32][sub = p/16][part = (x%32)/8][row = p%16][e = x%8]
+//   f32:  [step = x/16][sub = p/16][part = (x%16)/4][row = p%16][e = x%4]
+// V, element (p, x) of a block:
+//   bf16, 32 positions: [dt = x/16][g = (p%16)/4][m = x%16][e = 4*(p/16) + p%4]
+//   f32,  16 positions: [dt = x/16][g = p/4][m = x%16][j = p%4]
 template <typename T> struct KvTile;
 
 template <> struct KvTile<uint16_t> {
     static constexpr int BLK = 32;
+    static constexpr int KCH = 64;
     __host__ __device__ static inline int64_t k_off(int64_t pos, int x, int D) {
-        const int64_t blk = pos / 32;
-        const int p = (int)(pos % 32);
-        return blk * 32 * D + (((int64_t)(x / 32) * 2 + p / 16) * 4 + (x % 32) / 8) * 128 + (p % 16) * 8 + (x % 8);
+        const int64_t ch = pos / 64;
+        const int p = (int)(pos % 64);
+        return ch * 64 * D + (((int64_t)(x / 32) * 4 + p / 16) * 4 + (x % 32) / 8) * 128 + (p % 16) * 8 + (x % 8);
     }
     __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
         const int64_t blk = pos / 32;
@@ -82,10 +85,11 @@ template <> struct KvTile<uint16_t> {
 
 template <> struct KvTile<float> {
     static constexpr int BLK = 16;
+    static constexpr int KCH = 64;
     __host__ __device__ static inline int64_t k_off(int64_t pos, int x, int D) {
-        const int64_t blk = pos / 16;
-        const int p = (int)(pos % 16);
-        return blk * 16 * D + ((int64_t)(x / 4) * 16 + p) * 4 + (x % 4);
+        const int64_t ch = pos / 64;
+        const int p = (int)(pos % 64);
+        return ch * 64 * D + (((int64_t)(x / 16) * 4 + p / 16) * 4 + (x % 16) / 4) * 64 + (p % 16) * 4 + (x % 4);
     }
     __host__ __device__ static inline int64_t v_off(int64_t pos, int x, int D) {
         const int64_t blk = pos / 16;
@@ -94,19 +98,8 @@ template <> struct KvTile<float> {
     }
 };
 
-// Ticket records of the merge that runs inside the split-K launch: two sets of `cap` 64-bit
-// words; launches alternate between the sets and each clears what the other set's last user
-// touched (sdpa_decode.hip).  Host-side bookkeeping of one stream's launches.
-struct TicketRecords {
-    unsigned long long *dev = nullptr;
-    size_t cap = 0;            // records per set
-    int cur = 0;               // set the next launch uses
-    size_t used[2] = {0, 0};   // records of each set that may be non-zero
-};
-
-// Polls a helper workgroup of the in-launch merge makes before it gives up (about 0.1 us of
-// sleep plus one read of the record each).
-static constexpr int kDefaultMergeWait = 24;
+// positions the planes are padded to (whole K chunks, which are whole V blocks)
+static constexpr int kKvChunk = 64;
 
 // ---- context ----------------------------------------------------------------
 struct LinearWeights {
@@ -162,7 +155,7 @@ struct Ctx {
     int32_t step_launches = 2;   // launches of mfa_full_attn_step: 2 (prologue inside the attention launch) or 3
     float *qg_chunk = nullptr;   // the same for a chunk of tokens (mfa_prefill_full_attn), grown on demand
     size_t qg_chunk_elems = 0;
-    int64_t cap_pad = 0;        // kv capacity rounded up to whole blocks
+    int64_t cap_pad = 0;        // kv capacity rounded up to whole K chunks
     size_t plane_elems = 0;     // elements of one (layer, K|V, kv head) plane
     // split-K workspace
     float *part_o = nullptr;
@@ -170,9 +163,6 @@ struct Ctx {
     size_t part_o_elems = 0, part_ml_elems = 0;
     int32_t forced_splits = 0;
     int32_t partial_only = 0;
-    TicketRecords tickets;      // of the merge inside the split-K launch
-    int32_t merge_wait = kDefaultMergeWait;
-    int32_t separate_merge = 1;   // the merge is a launch of its own unless mfa_set_merge asks otherwise
     // scratch of the Gated-DeltaNet chunk kernels (grown on demand)
     float *gdn_scratch = nullptr;
     size_t gdn_scratch_elems = 0;
@@ -216,9 +206,6 @@ struct SdpaWorkspace {
     float *part_o;
     float *part_ml;
     size_t part_o_elems, part_ml_elems;
-    TicketRecords *tickets = nullptr;   // null: the merge is always a second launch
-    int merge_wait = 0;                 // polls of a helper workgroup before it gives up
-    int separate_merge = 1;             // 0: merge inside the split-K launch (needs tickets)
 };
 bool sdpa_shape_supported(int kv_dtype, int head_dim);
 // Number of splits the launcher will use (for workspace sizing pass kv_len = capacity).

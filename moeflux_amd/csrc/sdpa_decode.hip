@@ -6,69 +6,42 @@
 // crates/moeflux/src/riir/linear_attn_forward.rs:850-902) and its CPU fallback
 // sdpa_cpu (crates/moeflux/src/riir/sdpa.rs:63-172) with two launches:
 //
-//   sdpa_partial_kernel  grid (splits, head groups, kv heads), W = 4 or 8 waves.
-//     The cache is consumed in super-blocks of W position blocks.  The up to 16
-//     query heads that share the kv head are the N dimension of the matrix
-//     instruction, so lane%16 is the head index throughout:
-//       phase 1  wave w:  S^T[pos, head] = K[pos, :] . Q[head, :] for its own
-//                block (the block's K is one contiguous run, read as 1 KiB
-//                wave loads straight into MFMA operand registers); the tile
-//                maxima meet in LDS, every wave forms the same running max,
-//                and the probabilities go to LDS already in operand order.
-//       phase 2  wave w:  O^T[d, head] += V^T[d, pos] . P^T[pos, head] for ALL W
-//                blocks of the super-block but only its own D/(16 W) output
-//                tiles, so no wave ever holds more than its slice of O and
-//                nothing has to be summed across waves at the end.
-//     Each byte of K and V is read exactly once.  All loads of a super-block
-//     are issued before its first use (the query's first of all, because
-//     loads return in order); the next super-block's K is requested when the
-//     K registers free up after phase 1, its V after phase 2.
-//     bf16 caches use v_mfma_f32_16x16x32_bf16 with the f32 query and the f32
-//     probabilities each split into a bf16 high and low part (two
-//     instructions, products exact to ~2^-17); f32 caches use
-//     v_mfma_f32_16x16x4_f32.  The query is pre-multiplied by scale*log2 e so a
-//     probability is one v_exp_f32.  One (max, sum, O[16, D]) partial per
-//     workgroup is written.
-//   The log-sum-exp merge of the partials, the normalisation and the sigmoid gate
-//   run in the same launch: every workgroup takes a ticket of its row group when its
-//   partial is visible device-wide, and the one that draws the last ticket (helped,
-//   when the group has many splits, by workgroups that arrived a moment earlier and
-//   looked on for a bounded time) combines the group's partials.  No workgroup ever
-//   depends on another one making progress.  sdpa_merge_kernel / sdpa_merge_few_kernel
-//   are the same merge as a launch of its own (the latent-cache attention uses them).
+//   sdpa_partial_kernel  grid (splits, 16-row groups, kv heads), 4 waves.
+//     A workgroup streams its share of the cache: K and V pass through a ring of eight 1 KiB
+//     loads per wave, each consumed by the matrix core as it arrives and replaced by the next
+//     request, so a CU keeps 32 KiB in flight and its four waves, reading side by side, sweep
+//     one contiguous run of memory (measured on 64 MiB: 10.8 us per launch in this pattern,
+//     12.8 us with a workgroup's whole share requested at once, 11.5-12 us with one contiguous
+//     run per wave).  The up to 16 query heads that share the kv head are the N dimension of the
+//     matrix instruction, so lane % 16 is the head index throughout.  The cache is consumed in
+//     passes of up to G chunks of 64 positions:
+//       K phase  wave w owns the 16-position sub-tile w of every chunk:
+//                S^T[pos, head] += K[pos, k-step] . Q[head, k-step] per load, the query operands
+//                in registers; while the last K loads are consumed the first V loads go out.
+//       exchange the waves' maxima meet in LDS, every wave forms the same running max, and
+//                the probabilities go to LDS already in operand order (two LDS barriers per
+//                pass; they wait for LDS only, the ring stays in flight).
+//       V phase  wave w owns the output tiles w, w + 4, ...:
+//                O^T[d, head] += V^T[d, pos] . P^T[pos, head] per load, over all positions of
+//                the pass, so nothing is summed across waves at the end; while the last V
+//                loads are consumed the next pass's first K loads go out.
+//     Each byte of K and V is read exactly once.  bf16 caches use v_mfma_f32_16x16x32_bf16
+//     with the f32 query and the f32 probabilities each split into a bf16 high and low part
+//     (two instructions, products exact to ~2^-17); f32 caches use v_mfma_f32_16x16x4_f32.
+//     The query is pre-multiplied by scale*log2 e so a probability is one v_exp_f32.  One
+//     (max, sum, O[16, D]) partial per workgroup is written.
+//   sdpa_merge_kernel / sdpa_merge_few_kernel: the log-sum-exp merge of the partials, the
+//     normalisation and the sigmoid gate.
 #include "attn_prologue.h"
 #include "sdpa_merge.h"
 
 namespace mfa {
 
 static constexpr int kMaxSplits = 1024;
+static constexpr int kWaves = 4;     // waves of a split-K workgroup
 
 // part_o:  [kv head][head group][split][16 heads][D]
 // part_ml: [kv head][head group][split][2][16]   (max in log2 units, then sum)
-// The merge inside the split-K launch.  A row group's record is one 64-bit word, zero when the
-// launch starts: arrivals in the high half, claimed chunks of the group's output in the low half.
-//   * A workgroup makes its partial visible device-wide (release fence), then adds 1 to the
-//     arrivals with one device-scope atomic; the value that comes back is its ticket.  The one
-//     that draws the last ticket knows every partial of the group is complete.
-//   * Few splits (<= 16): that workgroup merges the whole group, all requests in flight at once.
-//   * Many splits: the group's output is cut into chunks and the workgroups of the first splits
-//     are helpers: a helper claims chunk `split` in the same atomic that takes its ticket, then
-//     reads the record a bounded number of times; when it sees the last arrival it merges its
-//     chunk.  A helper that gives up hands the chunk back (one atomic; should the last arrival
-//     have come in between, it merges the chunk after all).  The last arrival merges every chunk
-//     nobody held when it arrived.  Each chunk has exactly one owner, who only starts once all
-//     partials are visible, and no workgroup waits without a bound: progress never depends on
-//     which workgroups are resident.
-//   * Records are never reset by the launch that uses them: launches alternate between two sets
-//     of records, and each launch zeroes the records the previous user of the other set touched.
-struct FusedMerge {
-    unsigned long long *rec;    // this launch's records [kv head][row group]; null: no merge in this launch
-    unsigned long long *zero;   // records of the other set to clear, [0, n_zero)
-    int n_zero;
-    int wait;                   // polls a helper makes before it gives up
-    const float *gate;
-    float *out;
-};
 
 // The attention prologue of one decode token inside the split-K launch
 // (full_attn_forward.rs:238-323: q/gate split, per-head RMS norms of q and k, rotation of the
@@ -87,6 +60,7 @@ struct StepPrologue {
     void *k_tiled, *v_tiled;   // the planes, to append to
     int token_split;           // the split whose workgroup also scores and appends the token
 };
+struct NoPrologue {};          // what the plain launch carries in its place
 
 // The query operands of the workgroup's 16 rows from the raw q projection: a group of
 // LPH = D / EPS lanes serves one head, lane j its channels [EPS j, EPS j + EPS), which is exactly
@@ -184,69 +158,111 @@ template <typename KV, int D, int NT> struct StepQuery {
     }
 };
 
-static constexpr int kFewSplits = 16;        // at most this many: merged by one workgroup in one go
-static constexpr int kMaxMergeChunks = 32;   // claim bits of a record
 
-template <typename KV, int D, int WAVES, bool STEP>
-__global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
+// LDS-only barrier: every LDS access of the wave has completed, then the workgroup meets.  Unlike
+// __syncthreads() it places no wait on the vector-memory counter, so the ring's loads stay in flight.
+__device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// 1 KiB loads a wave keeps in flight.  Eight (32 KiB per CU) is where a plain streaming read of 64 MiB
+// is fastest; the widest heads take sixteen, which also keeps the memory system busy while a
+// workgroup stages its query and exchanges its probabilities (bf16, head_dim 256, 32768 positions:
+// 13.2 us per launch with 8, 12.75 with 16, 12.9 with 32; 14.9 with 4).
+__host__ __device__ constexpr int ring_depth(bool bf16, int D) { return bf16 && D == 256 ? 16 : 8; }
+
+// Shape constants of the streaming kernel.  A pass takes NCH chunks; its K is NCH * NK loads per
+// wave, its V as many.  The unified sequence of a wave's loads (K of a pass, its V, K of the next
+// pass, ...) runs through the ring with load number i in slot i % R, which holds as long as a pass
+// is at least one ring of K (MINCH chunks) and two of its phases are whole rings (chunk counts that
+// are multiples of GRAN): then every pass begins at slot 0 again.
+template <typename KV, int D> struct Stream {
+    using W = Wave<KV, D>;
+    static constexpr int R = ring_depth(sizeof(KV) == 2, D);
+    static constexpr int CH = KvTile<KV>::KCH;              // positions of a K chunk
+    static constexpr int NK = W::KSTEPS;                    // K loads per chunk and wave (one per k-step)
+    static constexpr int VB = CH / W::BLK;                  // V blocks per chunk
+    static constexpr int TPW = W::NACC / kWaves;            // output tiles per wave
+    static constexpr int NV = VB * TPW;                     // V loads per chunk and wave
+    static constexpr int GRAN = (2 * NK) % R == 0 ? 1 : R / (2 * NK);   // chunk counts of a pass are multiples of this
+    static constexpr int MINCH = (R + NK - 1) / NK < GRAN ? GRAN : (R + NK - 1) / NK;   // chunks of the smallest pass
+    // A workgroup's share is streamed in passes of MAIN chunks until at most GMAX are left, which
+    // are one last pass: one exchange of maxima and probabilities per pass, and a share a little
+    // larger than the others' (a cache just past a multiple of the workgroups' shares) still is
+    // a single pass.
+    static constexpr int MAIN = sizeof(KV) == 2 ? 4 : 2;
+    static constexpr int GMAX = sizeof(KV) == 2 ? 6 : (D == 256 ? 2 : 3);
+    static constexpr int KCH_U4 = CH * D * (int)sizeof(KV) / 16;      // 16-byte words of a chunk of K
+    static constexpr int VBLK_U4 = W::BLK * D * (int)sizeof(KV) / 16;  // of a block of V
+    static_assert(NV == NK && W::NACC % kWaves == 0, "K and V of a chunk are the same number of loads");
+    static_assert(MAIN % GRAN == 0 && GMAX % GRAN == 0 && MAIN >= MINCH && GMAX - MAIN + GRAN >= MINCH,
+                  "every pass of a long share is a whole form");
+};
+
+// Calls f with the smallest of the chunk counts N, N + STEP, ... <= END that is at least `want`
+// (END if none is), as a compile-time constant.
+template <int N, int END, int STEP, typename F> __device__ __attribute__((always_inline)) inline void with_form(int want, F &&f) {
+    if constexpr (N + STEP > END) {
+        f(std::integral_constant<int, N>{});
+    } else {
+        if (want <= N) f(std::integral_constant<int, N>{});
+        else with_form<N + STEP, END, STEP>(want, f);
+    }
+}
+
+template <typename KV, int D, bool STEP>
+__global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     const KV *__restrict__ k_tiled, const KV *__restrict__ v_tiled, size_t plane_elems,
     const float *__restrict__ q, int hpk, int Hq, int n_tok, int64_t kv_len0,
-    int blocks_per_split, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml,
-    FusedMerge fm, StepPrologue sp) {
+    int units_base, int units_rem, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml,
+    std::conditional_t<STEP, StepPrologue, NoPrologue> sp) {
     using W = Wave<KV, D>;
-    constexpr int NACC = W::NACC;
-    constexpr int TPW = NACC / WAVES;  // output tiles owned by one wave
-    constexpr int NLOAD = W::NLOAD;
-    constexpr int NX = W::NX;
-    constexpr int NQ = (W::QSLOTS + WAVES * 64 - 1) / (WAVES * 64);  // query slots per thread
-    static_assert(NACC % WAVES == 0, "waves must divide the output tiles");
+    using S = Stream<KV, D>;
+    constexpr int NK = S::NK, NV = S::NV, TPW = S::TPW, VB = S::VB, kRing = S::R;
+    constexpr int NT = kWaves * 64;
+    constexpr int NQ = (W::QSLOTS + NT - 1) / NT;  // query slots per thread
     __shared__ uint4 qlds[W::QLDS_U4];
-    __shared__ uint4 pbuf[WAVES][W::P_U4][64];
-    __shared__ float sm[WAVES][16];
-    __shared__ float sl[WAVES][16];
+    __shared__ uint4 pbuf[S::GMAX * VB][W::P_U4][64];
+    __shared__ float sm[kWaves][16];
+    __shared__ float sl[kWaves][16];
     __shared__ float2 s_tab[STEP ? 128 : 1];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const int split = blockIdx.x, hg = blockIdx.y, kvh = blockIdx.z;
+    const int hg = blockIdx.y, kvh = blockIdx.z;
     const int nsplit = gridDim.x, nhg = gridDim.y;
+    const int split = blockIdx.x;
     // A decode step's launch: the workgroup of one split (the last, which has the fewest positions)
     // also norms and rotates the token's key, scores it against every query row of the group and
     // appends its row.  Uniform over the workgroup.
-    const bool with_new = STEP && split == sp.token_split;
+    bool with_new = false;
+    if constexpr (STEP) with_new = split == sp.token_split;
 
-    const int64_t blk_elems = (int64_t)W::BLK * D;
-    const KV *kplane = k_tiled + (size_t)kvh * plane_elems;
-    const KV *vplane = v_tiled + (size_t)kvh * plane_elems;
     const RowGroup rows{kvh, hg, hpk, Hq, n_tok, kv_len0};
     const int64_t limit = rows.limit(n);          // this lane's row sees positions [0, limit)
-    const int64_t limit_min = rows.limit_min();   // below it no row of the group is masked
-    const bool all_rows = rows.full();
-    const int64_t nblk = (rows.limit_max() + W::BLK - 1) / W::BLK;
-    const int64_t b0 = (int64_t)split * blocks_per_split;
-    int64_t b1 = b0 + blocks_per_split;
-    if (b1 > nblk) b1 = nblk;
+    // This split's chunks [c0, c1): the plan hands out units of GRAN chunks, the first units_rem
+    // splits one unit more than the others; a group whose rows end earlier stops there.
+    const int64_t nchunk = (rows.limit_max() + S::CH - 1) / S::CH;
+    const int64_t u0 = (int64_t)split * units_base + (split < units_rem ? split : units_rem);
+    const int64_t c0 = u0 * S::GRAN;
+    int64_t c1 = (u0 + units_base + (split < units_rem ? 1 : 0)) * S::GRAN;
+    if (c1 > nchunk) c1 = nchunk;
     const size_t pid = ((size_t)kvh * nhg + hg) * nsplit + split;
-    if (fm.rec && fm.n_zero > 0 && threadIdx.x == 0) {   // clear the other set's used records
-        const int nwg = gridDim.x * gridDim.y * gridDim.z;
-        for (int i = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; i < fm.n_zero; i += nwg)
-            fm.zero[i] = 0ull;
-    }
-    if (with_new && b0 >= b1) {
-        // no positions for this split (an empty cache): its partial weighs nothing, the token is all there is
-        if (wave == 0 && g == 0) {
-            const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, neg_inf()), mlb, n * 4, 0, kThrough);
-            __builtin_amdgcn_raw_buffer_store_b32(0u, mlb, (16 + n) * 4, 0, kThrough);
+    if constexpr (STEP) {
+        if (with_new && c0 >= c1) {
+            // no positions for this split (an empty cache): its partial weighs nothing, the token is all there is
+            if (wave == 0 && g == 0) {
+                const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, neg_inf()), mlb, n * 4, 0, kThrough);
+                __builtin_amdgcn_raw_buffer_store_b32(0u, mlb, (16 + n) * 4, 0, kThrough);
+            }
+            StepQuery<KV, D, NT> sq;
+            sq.request(sp, rows);
+            HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
+            __syncthreads();
+            sq.finish(sp, rows, qscale, plane_elems, true, qlds, nhg, s_tab);
+            return;
         }
-        StepQuery<KV, D, WAVES * 64> sq;
-        sq.request(sp, rows);
-        HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
-        __syncthreads();
-        sq.finish(sp, rows, qscale, plane_elems, true, qlds, nhg, s_tab);
-        return;
     }
-    if (b0 >= b1) {  // a split that lies wholly beyond what this group's rows may see
+    if (c0 >= c1) {  // a split that lies wholly beyond what this group's rows may see
         // Its rows of part_o stay unwritten: the merge gives a split whose maximum is -inf the
         // weight 0 by selection, so whatever bytes the workspace holds there never enter a sum.
         if (wave == 0 && g == 0) {
@@ -254,270 +270,188 @@ __global__ __launch_bounds__(WAVES * 64) void sdpa_partial_kernel(
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, neg_inf()), mlb, n * 4, 0, kThrough);
             __builtin_amdgcn_raw_buffer_store_b32(0u, mlb, (16 + n) * 4, 0, kThrough);
         }
-    } else {
+        return;
+    }
 
     // ---- requests, in the order they are needed (loads return in order) ---------
     // Every load below is unconditional (indices are clamped instead), so that the
     // compiler can count outstanding loads exactly and wait for the query without
     // waiting for the cache.
     float4 qraw[NQ][W::QRAW_F4];
-    StepQuery<KV, D, WAVES * 64> sq;
-    if (STEP) {
+    StepQuery<KV, D, NT> sq;
+    if constexpr (STEP) {
         sq.request(sp, rows);
-        __builtin_amdgcn_s_barrier();
     } else {
 #pragma unroll
         for (int i = 0; i < NQ; i++) {
-            int slot = threadIdx.x + i * WAVES * 64;
+            int slot = threadIdx.x + i * NT;
             if (slot >= W::QSLOTS) slot = W::QSLOTS - 1;
             W::load_q_slot(qraw[i], q, slot, rows);
         }
-        // A CU returns load data in request order across its waves: hold the bulk requests
-        // back until every wave's query request is queued, or a late wave's query would
-        // sit behind its siblings' cache blocks.
-        __builtin_amdgcn_s_barrier();
     }
-    uint4 kreg[NLOAD];
-    uint4 vreg[WAVES][TPW];
-    // loads [i0, i1) of this wave's K block of the super-block starting at sb
-    auto load_k_part = [&](int64_t sb, int i0, int i1) {
-        int64_t blk = sb + wave;
-        if (blk > b1 - 1) blk = b1 - 1;  // a wave without a block re-reads the last one and ignores it
-        const uint4 *p = (const uint4 *)(kplane + blk * blk_elems) + lane;
-#pragma unroll
-        for (int i = i0; i < i1; i++) kreg[i] = stream_load(p + i * 64);
+    // A CU returns load data in request order across its waves: hold the cache requests
+    // back until every wave's query request is queued, or a late wave's query would
+    // sit behind its siblings' cache data.
+    __builtin_amdgcn_s_barrier();
+
+    // Piece (k-step s, sub-tile `wave`) of a chunk's K and piece (tile 4t + wave) of a block's V
+    // are 16-byte word s * 256 (t * 256) + wave * 64 + lane of the chunk (block): the four waves'
+    // loads of one step are 4 KiB side by side, consecutive steps follow each other in memory.
+    const uint4 *kbase = reinterpret_cast<const uint4 *>(k_tiled + (size_t)kvh * plane_elems) + wave * 64 + lane;
+    const uint4 *vbase = reinterpret_cast<const uint4 *>(v_tiled + (size_t)kvh * plane_elems) + wave * 64 + lane;
+    const int64_t cmax = c1 - 1, vmax = c1 * VB - 1;   // requests past the split's end re-read its last chunk / block
+    auto k_load = [&](int64_t chunk, int s) {
+        const int64_t c = chunk < cmax ? chunk : cmax;
+        return stream_load(kbase + c * S::KCH_U4 + s * 256);
     };
-    auto load_k = [&](int64_t sb) { load_k_part(sb, 0, NLOAD); };
-    // V of blocks [j0, j1) of the super-block starting at sb
-    auto load_v = [&](int64_t sb, int j0, int j1) {
-#pragma unroll
-        for (int j = j0; j < j1; j++) {
-            int64_t blk = sb + j;
-            if (blk > b1 - 1) blk = b1 - 1;
-            const uint4 *p = (const uint4 *)(vplane + blk * blk_elems) + lane + (wave * TPW) * 64;
-#pragma unroll
-            for (int t = 0; t < TPW; t++) vreg[j][t] = stream_load(p + t * 64);
-        }
+    auto v_load = [&](int64_t blk, int t) {
+        const int64_t b = blk < vmax ? blk : vmax;
+        return stream_load(vbase + b * S::VBLK_U4 + t * 256);
     };
-    // A wave issues in order, and a CU accepts only so many outstanding loads: requesting
-    // all of V here would keep the wave stuck in the issue stage long after its K has
-    // arrived.  So only kVEarly blocks of V go out now, the rest once the scores are under way.
-    constexpr int kVEarly = WAVES / 4;
-    if (STEP) {
-        // Three quarters of the K block are requested first (measured against a quarter, half, all and
-        // none of it: 18.5 us per step against 20.1, 18.9, 19.1 and 20.3): enough to keep the memory pipeline full while
-        // the first wave forms the rotation table and every wave norms and rotates its share of
-        // the query (a wave cannot compute while its requests wait for room in the queue, which
-        // the full set would do for microseconds).  The rest follows when the query is in LDS.
-        load_k_part(b0, 0, NLOAD * 3 / 4);
+    uint4 ring[kRing];
+    constexpr int kHead = kRing < 8 ? kRing : 8;   // of the ring's first requests, those made before the query is staged
+#pragma unroll
+    for (int i = 0; i < kHead; i++) {
+        ring[i] = k_load(c0 + i / NK, i % NK);
+        __builtin_amdgcn_sched_barrier(0);   // in ring order: loads return in the order of their requests
+    }
+
+    if constexpr (STEP) {
         HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
-        __syncthreads();
+        lds_barrier();
         sq.finish(sp, rows, qscale, plane_elems, with_new, qlds, nhg, s_tab);
-        load_k_part(b0, NLOAD * 3 / 4, NLOAD);
-        load_v(b0, 0, kVEarly);
     } else {
-        load_k(b0);
-        load_v(b0, 0, kVEarly);
 #pragma unroll
         for (int i = 0; i < NQ; i++) {
-            const int slot = threadIdx.x + i * WAVES * 64;
+            const int slot = threadIdx.x + i * NT;
             if (slot < W::QSLOTS) W::store_q_slot(qlds, qraw[i], slot, qscale);
         }
     }
-    __syncthreads();
+#pragma unroll
+    for (int i = kHead; i < kRing; i++) {
+        ring[i] = k_load(c0 + i / NK, i % NK);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    lds_barrier();
+    uint4 qr[W::QREGS];
+#pragma unroll
+    for (int i = 0; i < W::QREGS; i++) qr[i] = qlds[i * 64 + lane];
 
     f32x4 o[TPW];
 #pragma unroll
     for (int t = 0; t < TPW; t++) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = neg_inf(), l_run = 0.f;
 
-    // One super-block.  `more` is a compile-time constant at both call sites so that
-    // each path has a fixed sequence of loads.
-    auto super_block = [&](int64_t sb, auto more_tag, auto first_tag) {
-        constexpr bool more = decltype(more_tag)::value;
-        constexpr int v_issued = decltype(first_tag)::value ? kVEarly : WAVES;  // V blocks already requested
-        const int64_t blk = sb + wave;
-        const bool have = blk < b1;
-        // ---- phase 1: this wave's block of scores ------------------------------
-        float x[NX];
+    // One pass over NCH chunks starting at chunk cb; the ring holds the pass's first K loads.
+    // NCH and MORE (another pass follows) are compile-time constants at every call site, so each
+    // form is a fixed sequence of loads.
+    auto pass = [&](int64_t cb, auto nch_tag, auto more_tag) __attribute__((always_inline)) {
+        constexpr int NCH = decltype(nch_tag)::value;
+        constexpr bool MORE = decltype(more_tag)::value;
+        constexpr int KL = NCH * NK, VL = NCH * NV;
+        constexpr int VO = KL % kRing;   // ring slot of the pass's first V load
+        static_assert(KL >= kRing && (KL + VL) % kRing == 0, "a ring of K at least, and the next pass begins at slot 0");
+        // ---- K phase: this wave's sub-tile of every chunk ----------------------------------
+        f32x4 sc[NCH];
+#pragma unroll
+        for (int c = 0; c < NCH; c++) sc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KL; i++) {
+            sc[i / NK] = W::score_step(ring[i % kRing], qr, i % NK, sc[i / NK]);
+            if (i + kRing < KL) ring[i % kRing] = k_load(cb + (i + kRing) / NK, (i + kRing) % NK);
+            else ring[i % kRing] = v_load(cb * VB + (i + kRing - KL) / TPW, (i + kRing - KL) % TPW);
+            // the request stays here, a ring's length ahead of its use (left alone the scheduler
+            // sinks it to just before the use, and the ring runs one or two deep)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        float x[4 * NCH];
         float m_loc = neg_inf();
-        {
-            typename W::Scores sc;
-            W::scores(kreg, qlds, lane, sc);
-            W::unpack(sc, x);
-        }
-        if (v_issued < WAVES) load_v(sb, v_issued, WAVES);
-        if (more) load_k(sb + WAVES);  // the K registers are free again
-        if (!have || !all_rows || (blk + 1) * W::BLK > limit_min) {  // a block some row must not see in full
 #pragma unroll
-            for (int e = 0; e < NX; e++)
-                if (!have || W::pos_of(blk, g, e) >= limit) x[e] = neg_inf();
-        }
+        for (int c = 0; c < NCH; c++) {
+            // positions 4g .. 4g+3 of sub-tile `wave` of chunk cb + c: the first `nv` of them exist for
+            // this lane's row (none in a chunk past the split's end, whose loads re-read the last one)
+            const int64_t chunk = cb + c;
+            int64_t room = limit - (chunk * S::CH + 16 * wave + 4 * g);
+            if (chunk >= c1) room = 0;
+            const int nv = room < 0 ? 0 : room > 4 ? 4 : (int)room;
 #pragma unroll
-        for (int e = 0; e < NX; e++) m_loc = fmaxf(m_loc, x[e]);
+            for (int r = 0; r < 4; r++) {
+                x[4 * c + r] = r < nv ? sc[c][r] : neg_inf();
+                m_loc = fmaxf(m_loc, x[4 * c + r]);
+            }
+        }
         m_loc = fmaxf(m_loc, lane_xor(m_loc, 16));
         m_loc = fmaxf(m_loc, lane_xor(m_loc, 32));
         if (g == 0) sm[wave][n] = m_loc;
-        __syncthreads();
+        lds_barrier();
         float m_new = m_run;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) m_new = fmaxf(m_new, sm[w][n]);
+        for (int w = 0; w < kWaves; w++) m_new = fmaxf(m_new, sm[w][n]);
         // a row that has seen nothing yet (its limit lies further on, or it is padding) keeps -inf
         const float m_ref = (m_new == neg_inf()) ? 0.f : m_new;
         const float alpha = fast_exp2(m_run - m_ref);
         m_run = m_new;
         float psum = 0.f;
-        {
-            float e[NX];
 #pragma unroll
-            for (int i = 0; i < NX; i++) {
-                e[i] = fast_exp2(x[i] - m_ref);  // 0 for masked positions
-                psum += e[i];
+        for (int c = 0; c < NCH; c++) {
+            float e[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                e[r] = fast_exp2(x[4 * c + r] - m_ref);  // 0 for masked positions
+                psum += e[r];
             }
-            uint4 p[W::P_U4];
-            W::pack_probs(e, p);
-#pragma unroll
-            for (int i = 0; i < W::P_U4; i++) pbuf[wave][i][lane] = p[i];
+            // sub-tile `wave` of chunk c is half wave % 2 of V block 2c + wave / 2 (bf16), V block 4c + wave (f32)
+            W::store_probs(pbuf[c * VB + (wave * VB) / 4], lane, wave & 1, e);
         }
         l_run = l_run * alpha + psum;
-        __syncthreads();
-        // ---- phase 2: every block of the super-block, this wave's output tiles --
+        lds_barrier();
+        // ---- V phase: every position of the pass, this wave's output tiles -----------------
         if (__any(alpha != 1.0f)) {  // the running max moved
 #pragma unroll
             for (int t = 0; t < TPW; t++) {
                 o[t][0] *= alpha; o[t][1] *= alpha; o[t][2] *= alpha; o[t][3] *= alpha;
             }
         }
+        uint4 p[W::P_U4];
 #pragma unroll
-        for (int j = 0; j < WAVES; j++) {
-            // a block past the end contributes probabilities that are all zero
-            uint4 p[W::P_U4];
+        for (int i = 0; i < VL; i++) {
+            if (i % TPW == 0) {
 #pragma unroll
-            for (int i = 0; i < W::P_U4; i++) p[i] = pbuf[j][i][lane];
-#pragma unroll
-            for (int t = 0; t < TPW; t++) o[t] = W::pv(vreg[j][t], p, o[t]);
+                for (int j = 0; j < W::P_U4; j++) p[j] = pbuf[i / TPW][j][lane];
+            }
+            o[i % TPW] = W::pv(ring[(VO + i) % kRing], p, o[i % TPW]);
+            if (i + kRing < VL) ring[(VO + i) % kRing] = v_load(cb * VB + (i + kRing) / TPW, (i + kRing) % TPW);
+            else if (MORE) ring[(VO + i) % kRing] = k_load(cb + NCH + (i + kRing - VL) / NK, (i + kRing - VL) % NK);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (more) load_v(sb + WAVES, 0, WAVES);
     };
-    if (b0 + WAVES < b1) {
-        super_block(b0, std::true_type{}, std::true_type{});
-        int64_t sb = b0 + WAVES;
-        for (; sb + WAVES < b1; sb += WAVES) super_block(sb, std::true_type{}, std::false_type{});
-        super_block(sb, std::false_type{}, std::false_type{});
-    } else {
-        super_block(b0, std::false_type{}, std::true_type{});
-    }
+    int64_t cb = c0;
+    for (; c1 - cb > S::GMAX; cb += S::MAIN) pass(cb, std::integral_constant<int, S::MAIN>{}, std::true_type{});
+    // the last pass, in the smallest form that holds what is left (a form's chunks past the split's
+    // end re-read its last chunk and are masked)
+    with_form<S::MINCH, S::GMAX, S::GRAN>((int)(c1 - cb), [&](auto nch) __attribute__((always_inline)) { pass(cb, nch, std::false_type{}); });
 
     // ---- one partial per workgroup -----------------------------------------------
     l_run += lane_xor(l_run, 16);
     l_run += lane_xor(l_run, 32);
     if (g == 0) sl[wave][n] = l_run;
-    // stores that go through to memory: the partial is read by whichever workgroup merges the group
     const __amdgpu_buffer_rsrc_t ob = buffer_of(part_o + pid * 16 * D);
 #pragma unroll
     for (int t = 0; t < TPW; t++) {
-        // tile dt, lane group g, element i is channel 16 dt + 4g + i of head n
+        // tile dt = 4t + wave, lane group g, element i is channel 16 dt + 4g + i of head n
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o[t]), ob,
-                                               (n * D + 16 * (wave * TPW + t) + 4 * g) * 4, 0, kThrough);
+                                               (n * D + 16 * (kWaves * t + wave) + 4 * g) * 4, 0, kThrough);
     }
-    __syncthreads();
+    lds_barrier();
     if (wave == 0 && g == 0) {
         float lsum = 0.f;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) lsum += sl[w][n];
+        for (int w = 0; w < kWaves; w++) lsum += sl[w][n];
         const __amdgpu_buffer_rsrc_t mlb = buffer_of(part_ml + pid * 32);
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, m_run), mlb, n * 4, 0, kThrough);
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, lsum), mlb, (16 + n) * 4, 0, kThrough);
     }
-    }  // a split with positions
-
-    if (!fm.rec) return;   // partials only (uniform over the launch)
-
-    // ---- ticket, and the merge by whoever it falls to -----------------------------------------
-    constexpr int TEAMS = WAVES / 4;                 // 256-thread teams of the many-split merge
-    constexpr int PER_ROW = D / 64;                  // 64-output units per row
-    constexpr int UNITS = 16 * PER_ROW;              // units of a row group
-    __shared__ float4 acc4[TEAMS][2][16][16];
-    __shared__ unsigned int s_own;                   // chunks this workgroup merges (bit set), 0: none
-    const size_t pid0 = ((size_t)kvh * nhg + hg) * nsplit;
-    const MergeOut mo{fm.gate, fm.out, hpk, Hq, n_tok, D, D, nullptr, nullptr, 0, nhg};
-    const bool few = nsplit <= kFewSplits;
-    // chunks of the many-split merge: a power of two, at most one per split, at most 32, and
-    // not finer than what the workgroup's teams merge in one pass
-    int nchunks = UNITS / TEAMS < kMaxMergeChunks ? UNITS / TEAMS : kMaxMergeChunks;
-    while (nchunks > nsplit) nchunks >>= 1;
-    const bool helper = !few && split < nchunks;
-
-    // The partial was written with stores that go through to memory: once every wave has counted
-    // its own off it is visible device-wide, and the ticket is taken after that.
-    wait_for_stores();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned long long *rec = fm.rec + (size_t)kvh * nhg + hg;
-        const unsigned long long one = 1ull << 32, bit = helper ? (1ull << split) : 0ull;
-        const unsigned long long old = __hip_atomic_fetch_add(rec, one + bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned int own = 0;
-        if ((int)(old >> 32) == nsplit - 1) {
-            // the last arrival: every chunk no helper held at this moment (its own included)
-            const unsigned int all = few ? 1u : (nchunks == 32 ? 0xffffffffu : (1u << nchunks) - 1u);
-            own = all & ~(unsigned int)old;
-        } else if (helper) {
-            bool complete = false;
-            for (int i = 0; i < fm.wait && !complete; i++) {
-                __builtin_amdgcn_s_sleep(2);
-                complete = (int)(__hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == nsplit;
-            }
-            if (!complete) {
-                // give the chunk back; if the last arrival has been in the meantime, it left the chunk to us
-                const unsigned long long was = __hip_atomic_fetch_add(rec, 0ull - bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                complete = (int)(was >> 32) == nsplit;
-            }
-            if (complete) own = (unsigned int)bit;
-        }
-        s_own = own;
-    }
-    __syncthreads();
-    unsigned int own = s_own;
-    if (own == 0) return;
-    // every split's partial is in memory from here on; the reader's loads go there for it
-    const PartialsThrough rd(part_o, part_ml, pid0, D);
-
-    if (few) {
-        // the whole group in passes of WAVES * UPW units, every request of a pass in flight at once
-        if (nsplit <= 8) {
-            constexpr int UPW = 8;
-            for (int u0 = 0; u0 < UNITS; u0 += WAVES * UPW)
-                merge_few_units<8, UPW>(rd, nsplit, kvh, hg, u0 + wave * UPW, UNITS, mo, lane);
-        } else {
-            constexpr int UPW = 4;
-            for (int u0 = 0; u0 < UNITS; u0 += WAVES * UPW)
-                merge_few_units<16, UPW>(rd, nsplit, kvh, hg, u0 + wave * UPW, UNITS, mo, lane);
-        }
-        return;
-    }
-    const int team = threadIdx.x >> 8, ttid = threadIdx.x & 255;
-    const int upc = UNITS / nchunks;                 // units of a chunk, consecutive: a power of two
-    while (own) {
-        const int c = __builtin_ctz(own);
-        own &= own - 1;
-        // a chunk's units lie in one row when upc <= PER_ROW, else it is whole rows; a team
-        // takes spans of up to two units (128 channels) of one row at a time
-        constexpr int SPAN = PER_ROW >= 2 ? 2 : 1;   // units per team pass, at most
-        const int span = upc / TEAMS < SPAN ? 1 : SPAN;
-        for (int u0 = c * upc; u0 < (c + 1) * upc; u0 += TEAMS * span) {
-            const int u = u0 + team * span;
-            const bool in = u < (c + 1) * upc;
-            const int nn = (in ? u : 0) / PER_ROW, c0 = ((in ? u : 0) % PER_ROW) * 64;
-            const int64_t orow = mo.row(kvh, hg * 16 + nn);
-            const bool active = in && orow >= 0;
-            if (span == 2)
-                merge_span<2>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team], D);
-            else
-                merge_span<1>(rd, nsplit, D, active, nn, c0, orow, fm.gate, fm.out, ttid, acc4[team], D);
-        }
-    }
 }
-
 
 // The token a decode step has just appended, as one more split of the merge (MergeOut), and
 // where the gate rows lie.
@@ -602,44 +536,66 @@ int launch_sdpa_merge(hipStream_t stream, const SdpaWorkspace &ws, int splits, i
 }
 
 bool sdpa_shape_supported(int kv_dtype, int head_dim) {
-    if (kv_dtype != MFA_KV_F32 && kv_dtype != MFA_KV_BF16) return false;
+    if (kv_dtype != MFA_KV_BF16 && kv_dtype != MFA_KV_F32) return false;
     return head_dim == 64 || head_dim == 128 || head_dim == 256;
 }
 
-static int blk_of(int kv_dtype) { return kv_dtype == MFA_KV_BF16 ? 32 : 16; }
+// chunks of a unit of the plan (Stream::GRAN)
+static int unit_chunks(int kv_dtype, int D) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
+    return (2 * nk) % ring == 0 ? 1 : ring / (2 * nk);
+}
 
-// Partition of the cache's position blocks over workgroups.  A workgroup has 8 waves
-// (super-blocks of 8 blocks) when that still gives every CU a workgroup, else 4;
-// head_dim 64 has only 4 output tiles, hence 4 waves.  n_tok > 1 (a prompt chunk)
-// multiplies the row groups, which already fill the machine, so the cache is split less.
+// chunks of the kernel's smallest pass (Stream::MINCH)
+static int min_pass_chunks(int kv_dtype, int D) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
+    const int m = (ring + nk - 1) / nk, g = unit_chunks(kv_dtype, D);
+    return m < g ? g : m;
+}
+
+// Partition of the cache over workgroups, in units of chunks of 64 positions (pairs of chunks at
+// head_dim 64 of a bf16 cache): `splits` workgroups per row group, the first `rem` of them `base + 1` units,
+// the others `base`.  The shares differ by at most one unit at every length, so the time of a
+// launch follows the length smoothly.  n_tok > 1 (a prompt chunk) multiplies the row groups,
+// which already fill the machine, so the cache is split less.
 struct SplitPlan {
     int splits;
-    int waves;
     int nhg;      // 16-row groups per kv head
-    int64_t bps;  // blocks per split
+    int base, rem;
 };
+
+// workgroups the plan aims at per (kv head, row group): every CU one, or two where a workgroup's
+// registers and LDS leave room and each still streams a few units
+static int64_t split_target(int Hq, int Hkv, int D, int64_t nhg, int64_t nunits, int num_cus, int wgs_per_cu) {
+    int64_t target = (int64_t)num_cus / ((int64_t)Hkv * nhg);
+    if (target < 1) target = 1;
+    if (wgs_per_cu > 1 && nunits >= 2 * wgs_per_cu * target) target *= wgs_per_cu;
+    if (target > kMaxSplits) target = kMaxSplits;
+    (void)Hq; (void)D;
+    return target;
+}
+
+static constexpr int g_wgs_per_cu = 1;
 
 static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
                              int num_cus, int forced) {
     const int hpk = Hq / Hkv;
     SplitPlan p;
     p.nhg = (int)(((int64_t)n_tok * hpk + 15) / 16);
-    const int64_t nblk = (kv_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
-    int64_t target = forced > 0 ? forced : (num_cus / ((int64_t)Hkv * p.nhg));
-    if (target < 1) target = 1;
-    // Up to head_dim 128 two 8-wave workgroups fit a CU (<= 128 registers): give every CU two
-    // where each still gets a whole pass of 8 blocks (f32, d=128, 32K: 25.6 -> 23.5 us).
-    if (forced <= 0 && D <= 128 && nblk >= 8 * 2 * target) target *= 2;
+    const int64_t nchunk = (kv_len + kKvChunk - 1) / kKvChunk;
+    const int U = unit_chunks(kv_dtype, D);
+    int64_t nunits = (nchunk + U - 1) / U;
+    if (nunits < 1) nunits = 1;
+    int64_t target = forced > 0 ? forced : split_target(Hq, Hkv, D, p.nhg, nunits, num_cus, g_wgs_per_cu);
     if (target > kMaxSplits) target = kMaxSplits;
-    p.bps = (nblk + target - 1) / target;
-    if (p.bps < 1) p.bps = 1;
-    p.waves = (p.bps >= 8 && D >= 128) ? 8 : 4;
-    // Whole super-blocks only (one block per wave and pass): a pass with idle waves costs as
-    // much as a full one, and fewer workgroups of full passes measured 12-18 % faster than
-    // one workgroup per CU with a ragged last pass (kv_len 20K-48K at 2 kv heads).
-    if (forced <= 0) p.bps = (p.bps + p.waves - 1) / p.waves * p.waves;
-    p.splits = (int)((nblk + p.bps - 1) / p.bps);
-    if (p.splits < 1) p.splits = 1;
+    if (target > nunits) target = nunits;
+    // a share smaller than the kernel's smallest pass would be padded with re-read chunks: the
+    // automatic plan rather takes fewer workgroups
+    const int64_t min_units = (min_pass_chunks(kv_dtype, D) + U - 1) / U;
+    if (forced <= 0 && target > 1 && nunits / target < min_units) target = nunits / min_units > 1 ? nunits / min_units : 1;
+    p.splits = (int)target;
+    p.base = (int)(nunits / target);
+    p.rem = (int)(nunits % target);
     return p;
 }
 
@@ -647,17 +603,11 @@ int sdpa_pick_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t kv_len, int n
     return plan_splits(kv_dtype, Hq, Hkv, D, 1, kv_len, num_cus, forced).splits;
 }
 
-// The most splits a decode launch makes at any cache length up to max_len: the plan's split count
-// is not monotonic in the length (whole passes per workgroup), its target is.
+// The most splits a decode launch makes at any cache length up to max_len: the plan's split
+// count never falls as the length grows.
 int sdpa_max_splits(int kv_dtype, int Hq, int Hkv, int D, int64_t max_len, int num_cus, int forced) {
     if (forced > 0) return forced < kMaxSplits ? forced : kMaxSplits;
-    const int hpk = Hq / Hkv;
-    const int64_t nhg = (hpk + 15) / 16, nblk = (max_len + blk_of(kv_dtype) - 1) / blk_of(kv_dtype);
-    int64_t target = num_cus / ((int64_t)Hkv * nhg);
-    if (target < 1) target = 1;
-    if (D <= 128 && nblk >= 8 * 2 * target) target *= 2;
-    if (target > kMaxSplits) target = kMaxSplits;
-    return (int)(target < nblk ? target : (nblk > 0 ? nblk : 1));
+    return plan_splits(kv_dtype, Hq, Hkv, D, 1, max_len > 0 ? max_len : 1, num_cus, 0).splits;
 }
 
 size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok) {
@@ -669,41 +619,21 @@ size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok) {
     return (size_t)Hkv * nhg * splits * 32;
 }
 
-template <typename KV, int D, int WAVES, bool STEP>
-static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v,
-                           size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                           int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
-                           const StepPrologue &sp) {
-    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, WAVES, STEP>), grid, dim3(WAVES * 64), 0, stream,
-                       (const KV *)k, (const KV *)v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                       qscale, po, pml, fm, sp);
-}
-
-template <typename KV, int D, bool STEP>
-static void launch_partial_w(int waves, hipStream_t stream, dim3 grid, const void *k, const void *v,
-                             size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                             int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
-                             const StepPrologue &sp) {
-    if constexpr (D >= 128) {
-        if (waves == 8) {
-            launch_partial<KV, D, 8, STEP>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps,
-                                           qscale, po, pml, fm, sp);
-            return;
-        }
-    }
-    launch_partial<KV, D, 4, STEP>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, qscale,
-                                   po, pml, fm, sp);
+template <typename KV, int D, bool STEP, typename SP>
+static void launch_partial(hipStream_t stream, dim3 grid, const void *k, const void *v, size_t plane_elems,
+                           const float *q, int hpk, int Hq, int n_tok, int64_t kv_len0, const SplitPlan &plan,
+                           float qscale, float *po, float *pml, const SP &sp) {
+    hipLaunchKernelGGL((sdpa_partial_kernel<KV, D, STEP>), grid, dim3(kWaves * 64), 0, stream, (const KV *)k,
+                       (const KV *)v, plane_elems, q, hpk, Hq, n_tok, kv_len0, plan.base, plan.rem, qscale, po, pml, sp);
 }
 
 // dtype and width dispatch of the split-K launch
-template <bool STEP>
-static void launch_partial_any(int kv_dtype, int D, int waves, hipStream_t stream, dim3 grid, const void *k,
-                               const void *v, size_t plane_elems, const float *q, int hpk, int Hq, int n_tok,
-                               int64_t kv_len0, int bps, float qscale, float *po, float *pml, const FusedMerge &fm,
-                               const StepPrologue &sp) {
-#define MFA_LAUNCH(KV, DD)                                                                                  \
-    launch_partial_w<KV, DD, STEP>(waves, stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, bps, \
-                                   qscale, po, pml, fm, sp)
+template <bool STEP, typename SP>
+static void launch_partial_any(int kv_dtype, int D, hipStream_t stream, dim3 grid, const void *k, const void *v,
+                               size_t plane_elems, const float *q, int hpk, int Hq, int n_tok, int64_t kv_len0,
+                               const SplitPlan &plan, float qscale, float *po, float *pml, const SP &sp) {
+#define MFA_LAUNCH(KV, DD) \
+    launch_partial<KV, DD, STEP>(stream, grid, k, v, plane_elems, q, hpk, Hq, n_tok, kv_len0, plan, qscale, po, pml, sp)
     if (kv_dtype == MFA_KV_BF16) {
         if (D == 64) MFA_LAUNCH(uint16_t, 64);
         else if (D == 128) MFA_LAUNCH(uint16_t, 128);
@@ -721,6 +651,22 @@ bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim) {
     return head_rotor_applies(kv_dtype, D, rotary_dim);
 }
 
+// A plan that fits the workspace: an automatic split count shrinks to fit; one forced for a
+// single token is used as given or refused.
+static int fit_plan(SplitPlan &plan, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len, int num_cus,
+                    int forced_splits, const SdpaWorkspace &ws) {
+    auto fits = [&](const SplitPlan &p) {
+        return sdpa_workspace_o_elems(Hq, Hkv, D, p.splits, n_tok) <= ws.part_o_elems &&
+               sdpa_workspace_ml_elems(Hq, Hkv, p.splits, n_tok) <= ws.part_ml_elems;
+    };
+    plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
+    while ((forced_splits <= 0 || n_tok > 1) && plan.splits > 1 && !fits(plan))
+        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
+    if (!fits(plan)) return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
+    if (plan.nhg > 65535 || Hkv > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
+    return MFA_OK;
+}
+
 // One decode token of a full-attention layer from its raw projections in two launches: the
 // split-K launch norms and rotates the query heads itself, attends to the len0 positions the
 // cache holds, and the workgroup of the last split (the one with the fewest positions) also scores
@@ -734,21 +680,14 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
         return fail(MFA_ERR_SHAPE, "attention step: shape not supported by the two-launch form");
     if (len0 < 0 || pos < 0) return fail(MFA_ERR_INVALID, "attention step: negative position");
     const int hpk = Hq / Hkv;
-    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits);
-    while (forced_splits <= 0 && plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, 1) > ws.part_o_elems ||
-                                                     sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, 1) > ws.part_ml_elems))
-        plan = plan_splits(kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, (plan.splits + 1) / 2);
-    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, 1) > ws.part_o_elems ||
-        sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, 1) > ws.part_ml_elems)
-        return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
+    SplitPlan plan;
+    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits, ws));
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
-    const FusedMerge fm{nullptr, nullptr, 0, 0, nullptr, nullptr};
     const StepPrologue sp{q_proj, k_in, v_in, q_norm, k_norm, inv_freq, rotary_dim, eps, pos, len0, new_score,
                           k_tiled, v_tiled, plan.splits - 1};
     // rows see positions [0, len0): one token whose own position is not in the cache yet
-    launch_partial_any<true>(kv_dtype, D, plan.waves, stream, dim3(plan.splits, plan.nhg, Hkv), k_tiled, v_tiled,
-                             plane_elems, nullptr, hpk, Hq, 1, len0 - 1, (int)plan.bps, qscale, ws.part_o, ws.part_ml,
-                             fm, sp);
+    launch_partial_any<true>(kv_dtype, D, stream, dim3(plan.splits, plan.nhg, Hkv), k_tiled, v_tiled, plane_elems,
+                             nullptr, hpk, Hq, 1, len0 - 1, plan, qscale, ws.part_o, ws.part_ml, sp);
     MFA_HIP(hipGetLastError());
     const MergeExtra ex{2 * D, new_score, v_in, kv_dtype == MFA_KV_BF16 ? 1 : 0};
     launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, 1, q_proj + D, out, &ex);
@@ -768,41 +707,13 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
     if (n_tok <= 0 || kv_len < n_tok)
         return fail(MFA_ERR_INVALID, "sdpa: kv_len must be > 0 (got %lld for %d tokens)", (long long)kv_len, n_tok);
     const int hpk = Hq / Hkv;
-    SplitPlan plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
-    // never exceed the workspace: a split count shrinks to fit, except one forced for a single
-    // token, which is used as given or refused
-    while ((forced_splits <= 0 || n_tok > 1) && plan.splits > 1 && (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
-                               sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems))
-        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
-    if (sdpa_workspace_o_elems(Hq, Hkv, D, plan.splits, n_tok) > ws.part_o_elems ||
-        sdpa_workspace_ml_elems(Hq, Hkv, plan.splits, n_tok) > ws.part_ml_elems)
-        return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
-    if (plan.nhg > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
+    SplitPlan plan;
+    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits, ws));
     // scores are produced in log2 units: q is pre-multiplied by (1/sqrt(D)) * log2(e)
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
-    const int64_t kv_len0 = kv_len - n_tok;
-    dim3 grid(plan.splits, plan.nhg, Hkv);
-    // The merge runs inside this launch when the workspace carries ticket records for every row
-    // group; otherwise (or when asked for) it is a second launch.
-    FusedMerge fm{nullptr, nullptr, 0, 0, gate, out};
-    TicketRecords *tk = ws.tickets;
-    const size_t groups = (size_t)Hkv * plan.nhg;
-    const bool fused = !partial_only && !ws.separate_merge && tk && tk->dev && groups <= tk->cap;
-    if (fused) {
-        fm.rec = tk->dev + (size_t)tk->cur * tk->cap;
-        fm.zero = tk->dev + (size_t)(tk->cur ^ 1) * tk->cap;
-        fm.n_zero = (int)tk->used[tk->cur ^ 1];
-        fm.wait = ws.merge_wait;
-    }
-    launch_partial_any<false>(kv_dtype, D, plan.waves, stream, grid, k_tiled, v_tiled, plane_elems, q, hpk, Hq, n_tok,
-                              kv_len0, (int)plan.bps, qscale, ws.part_o, ws.part_ml, fm, StepPrologue{});
+    launch_partial_any<false>(kv_dtype, D, stream, dim3(plan.splits, plan.nhg, Hkv), k_tiled, v_tiled, plane_elems, q,
+                              hpk, Hq, n_tok, kv_len - n_tok, plan, qscale, ws.part_o, ws.part_ml, NoPrologue{});
     MFA_HIP(hipGetLastError());
-    if (fused) {   // this set is in use now, the other one is clean again
-        tk->used[tk->cur] = groups;
-        tk->used[tk->cur ^ 1] = 0;
-        tk->cur ^= 1;
-        return MFA_OK;
-    }
     if (partial_only) return MFA_OK;
     launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, n_tok, gate, out);
     MFA_HIP(hipGetLastError());

@@ -1,10 +1,8 @@
-// Log-sum-exp merge of split-K partials: the device code shared by the stand-alone merge kernels
-// and by the merge that the split-K attention kernel runs itself once a row group's last split
-// has arrived.
+// Log-sum-exp merge of split-K partials: the device code of the merge kernels.
 //
 // Partials of one row group (16 query rows that share a kv head) lie at
 //   part_o  [pid0 + split][16 rows][D]      part_ml [pid0 + split][2][16]  (max in log2 units, sum)
-// and are read through a reader (PartialsPlain or PartialsThrough, sdpa_wave.h) by indices
+// and are read through a reader (PartialsPlain, sdpa_wave.h) by indices
 // relative to the group's first split.  A row's result is  sum_s w_s O_s / sum_s w_s l_s  with  w_s = 2^(m_s - max_s m_s), times
 // the sigmoid of the row's gate.  A split whose maximum is -inf (no row of the group could see
 // its positions) gets the weight 0 by selection and its rows are never added, whatever bytes

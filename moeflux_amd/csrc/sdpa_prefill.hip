@@ -9,8 +9,8 @@
 // A workgroup is 4 waves; every wave owns RG groups of 16 query rows (rows of one kv
 // head: token-major, then the hpk query heads that share it) from start to end: its
 // query operands and its output tiles stay in registers and its soft-max needs no other
-// wave.  The workgroup walks the cache blocks that its rows may see; each block's K and V
-// (already in MFMA operand order in memory) is copied into LDS once by all 256 threads,
+// wave.  The workgroup walks the cache blocks (of V: 32 or 16 positions) that its rows may see; each
+// block's K and V (already in MFMA operand order in memory) is copied into LDS once by all 256 threads,
 // double buffered, and every wave takes its operands from there.  With RG = 2 an operand
 // read from LDS feeds two row groups.  Nothing is split along the cache, so the gated,
 // normalised output is written directly.
@@ -76,10 +76,18 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
         constexpr int s0 = st.value * PER_T;
         int64_t blk = it * KS + ks;
         if (blk > nblk - 1) blk = nblk - 1;
-        const uint4 *kp = (const uint4 *)(kplane + blk * blk_elems) + tid;
+        // K lies in chunks of 64 positions, a k-step's four 16-position sub-tiles side by side
+        // (KvTile): piece li of the block (SUBS sub-tiles per k-step) is piece
+        // (li / SUBS) * 4 + first sub-tile + li % SUBS of its chunk.
+        constexpr int VB = KvTile<KV>::KCH / W::BLK, SUBS = 4 / VB;
+        const uint4 *kc = (const uint4 *)(kplane + (blk / VB) * (int64_t)(KvTile<KV>::KCH * D)) + (tid & 63);
+        const int sub0 = (int)(blk % VB) * SUBS;
         const uint4 *vp = (const uint4 *)(vplane + blk * blk_elems) + tid;
 #pragma unroll
-        for (int i = 0; i < PER_T; i++) stage[s0 + i] = vec_load(i < K_T ? kp + i * SET : vp + (i - K_T) * SET);
+        for (int i = 0; i < PER_T; i++) {
+            const int li = (i * SET + tid) >> 6;   // i < K_T: the piece of K this thread copies
+            stage[s0 + i] = vec_load(i < K_T ? kc + (((li / SUBS) * 4 + sub0 + li % SUBS) << 6) : vp + (i - K_T) * SET);
+        }
     };
     auto commit = [&](int buf, auto st) __attribute__((always_inline)) {
         constexpr int s0 = st.value * PER_T;

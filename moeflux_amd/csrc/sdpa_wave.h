@@ -45,45 +45,24 @@ __device__ inline uint4 stream_load(const uint4 *p) {
     return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p)));
 }
 
-// Split-K partials cross from the workgroup that writes them to the one that merges them, which
-// may run on another XCD with an L2 of its own.  The writer uses stores that go through to
-// memory (scope bits sc0 sc1) and counts them off (s_waitcnt vmcnt(0), which the compiler places
-// for these buffer instructions as for any other) before it takes its ticket; the reader uses
-// loads with the same bits, which do not hit lines its own L2 may hold.  A device-scope release
-// fence over ordinary stores instead writes the whole L2 back, once per wave: measured at 22 us
-// for 256 workgroups of 16 KiB each, against 5 us with these stores.
+// Split-K partials are written with stores that go through to memory (scope bits sc0 sc1): they
+// are read by the merge launch, whose workgroups run on other XCDs with L2s of their own, and
+// leaving 4 MB of them dirty in the writers' L2s until the end of the launch, to be written back
+// in one burst, measured slower.
 static constexpr int kThrough = 16;   // cache policy of the buffer instructions: sc1 (device scope)
 __device__ inline __amdgpu_buffer_rsrc_t buffer_of(const void *base) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0xffffffff, 0x00020000);
 }
 
-// Every store this wave has issued has reached its destination (for stores with the bits above:
-// memory).  A workgroup-scope fence does not wait for vector-memory stores on this target.
-__device__ inline void wait_for_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-// Readers of one row group's partials, by element index relative to the group's first split:
+// Reader of one row group's partials, by element index relative to the group's first split:
 // rows at (split * 16 + row) * D + channel, statistics at split * 32 + row (+ 16 for the sum).
-struct PartialsPlain {   // a launch of its own: the kernel boundary made the partials visible
+struct PartialsPlain {
     const float *o, *ml;
     __device__ PartialsPlain(const float *part_o, const float *part_ml, size_t pid0, int D)
         : o(part_o + pid0 * 16 * D), ml(part_ml + pid0 * 32) {}
     __device__ float stat(int i) const { return ml[i]; }
     __device__ float row1(int i) const { return o[i]; }
     __device__ float4 row4(int i) const { return *(const float4 *)(o + i); }
-};
-struct PartialsThrough {   // inside the launch that wrote them
-    __amdgpu_buffer_rsrc_t o, ml;
-    __device__ PartialsThrough(const float *part_o, const float *part_ml, size_t pid0, int D)
-        : o(buffer_of(part_o + pid0 * 16 * D)), ml(buffer_of(part_ml + pid0 * 32)) {}
-    __device__ float stat(int i) const {
-        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ml, i * 4, 0, kThrough));
-    }
-    __device__ float row1(int i) const {
-        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(o, i * 4, 0, kThrough));
-    }
-    __device__ float4 row4(int i) const {
-        return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(o, i * 4, 0, kThrough));
-    }
 };
 
 // The 16 rows a workgroup serves.  Row rr = 16*hg + n of kv head kvh is query head
@@ -108,8 +87,9 @@ struct RowGroup {
     __device__ bool full() const { return hg * 16 + 15 < n_tok * hpk; }
 };
 
-// Per-dtype pieces of the kernel.  Common shape: a block's K is NLOAD 1 KiB loads,
-// its V is NACC = D/16 1 KiB loads, load `dt` of V being the 16-wide output tile dt.
+// Per-dtype pieces of the kernels.  Common shape: the K of a 16-position sub-tile is KSTEPS
+// 1 KiB pieces (one per k-step), a V block is NACC = D/16 1 KiB pieces, piece `dt` being the
+// 16-wide output tile dt.  (NLOAD: pieces of K that cover the positions of one V block.)
 template <typename KV, int D> struct Wave;
 
 // ---------------------------------------------------------------------------
@@ -201,6 +181,25 @@ template <int D> struct Wave<uint16_t, D> {
                 sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s + 1]), sc.s[sub], 0, 0, 0);
             }
         }
+    }
+
+    // One 1 KiB piece of K (16 positions x the 32 channels of k-step s) against the query
+    // operands in registers: the piece's share of S^T[16 positions, 16 rows].
+    __device__ static f32x4 score_step(uint4 kpiece, const uint4 (&qr)[QREGS], int s, f32x4 acc) {
+        const bf16x8 a = as_bf16x8(kpiece);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s + 1]), acc, 0, 0, 0);
+        return acc;
+    }
+    // The probabilities of one 16-position sub-tile (lane (n, g): positions 4g .. 4g+3 of query
+    // row n) as this lane's half of the value product's operand: the sub-tile is half `h` of a
+    // 32-position V block, whose operand slots 4h .. 4h+3 of lane group g are those positions.
+    __device__ static void store_probs(uint4 (*pblk)[64], int lane, int h, const float (&e)[4]) {
+        uint2 hi, lo;
+        split_pair(e[0], e[1], hi.x, lo.x);
+        split_pair(e[2], e[3], hi.y, lo.y);
+        reinterpret_cast<uint2 *>(&pblk[0][lane])[h] = hi;
+        reinterpret_cast<uint2 *>(&pblk[1][lane])[h] = lo;
     }
 
     static constexpr int NX = 8;  // scores per lane: row 4g+i of sub-tile `sub` is position 16*sub + 4g + i
@@ -298,6 +297,21 @@ template <int D> struct Wave<float, D> {
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, sc.s, 0, 0, 0);
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, sc.s, 0, 0, 0);
         }
+    }
+
+    // One 1 KiB piece of K (16 positions x the 16 channels of k-step s).
+    __device__ static f32x4 score_step(uint4 kpiece, const uint4 (&qr)[QREGS], int s, f32x4 acc) {
+        const float4 a = __builtin_bit_cast(float4, kpiece);
+        const float4 b = __builtin_bit_cast(float4, qr[s]);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
+        return acc;
+    }
+    // A 16-position sub-tile is one V block: the four probabilities are the lane's operand.
+    __device__ static void store_probs(uint4 (*pblk)[64], int lane, int, const float (&e)[4]) {
+        pblk[0][lane] = __builtin_bit_cast(uint4, float4{e[0], e[1], e[2], e[3]});
     }
 
     static constexpr int NX = 4;  // row 4g+i is position 4g + i

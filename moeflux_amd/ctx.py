@@ -138,11 +138,6 @@ class Ctx:
     def set_num_splits(self, n: int):
         _chk(self.lib.mfa_set_num_splits(self.h, n), "mfa_set_num_splits")
 
-    def set_merge(self, in_launch: bool = False, helper_polls: int = -1):
-        """How split-K partials are combined: as a second launch (default) or inside the
-        attention launch; helper_polls bounds how long early workgroups look on (-1: default)."""
-        _chk(self.lib.mfa_set_merge(self.h, int(in_launch), helper_polls), "mfa_set_merge")
-
     def set_step_launches(self, launches: int):
         """Launches of full_attn_step: 2 (prologue inside the attention launch) or 3."""
         _chk(self.lib.mfa_set_step_launches(self.h, launches), "mfa_set_step_launches")

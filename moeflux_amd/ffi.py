@@ -42,7 +42,6 @@ SIGNATURES = {
     "mfa_set_linear_weights": (C.c_int, [vp, i32, u16p, f32p, u16p, u16p]),
     "mfa_set_num_splits": (C.c_int, [vp, i32]),
     "mfa_set_partial_only": (C.c_int, [vp, i32]),
-    "mfa_set_merge": (C.c_int, [vp, i32, i32]),
     "mfa_set_step_launches": (C.c_int, [vp, i32]),
     "mfa_host_alloc": (vp, [C.c_int64]),
     "mfa_host_free": (None, [vp]),

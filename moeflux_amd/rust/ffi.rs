@@ -109,7 +109,6 @@ extern "C" {
     // tuning and measurement
     pub fn mfa_set_num_splits(ctx: *mut mfa_ctx, num_splits: i32) -> c_int;
     pub fn mfa_set_partial_only(ctx: *mut mfa_ctx, on: i32) -> c_int;
-    pub fn mfa_set_merge(ctx: *mut mfa_ctx, in_launch: i32, helper_polls: i32) -> c_int;
     pub fn mfa_set_step_launches(ctx: *mut mfa_ctx, launches: i32) -> c_int;
     pub fn mfa_host_alloc(bytes: i64) -> *mut c_void;
     pub fn mfa_host_free(p: *mut c_void);

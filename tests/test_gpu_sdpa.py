@@ -136,53 +136,34 @@ def test_ctx_append_decode_and_split_invariance(mfa, oracle, bf16):
 def test_merge_of_several_hundred_splits(mfa, oracle, bf16):
     """More splits than the 256 whose statistics the merge keeps in registers (the rest are read
     in loops), and more than the 128 whose rows a thread requests up front: forced split counts
-    of 300, 512 and 1024 over a cache long enough to give every split a block."""
-    Hq, Hkv, d, L = 8, 1, 64, 17000
+    of 300, 512 and 1024 over a cache long enough to give every split a unit of the kernel's work
+    (64 positions of an f32 cache, 128 of a bf16 cache at this head width, so the plans end at 625
+    and 547 splits).  The oracle's sequential f32 sums over tens of thousands of positions are
+    themselves 1e-5 from exact, so the kernel is also held to a float64 evaluation."""
+    Hq, Hkv, d = 8, 1, 64
+    L = 70000 if bf16 else 40000
     q, g, k, v = sdpa_random_inputs(71, Hq, Hkv, d, L, bf16=bf16)
     kf = oracle.bf16_to_f32(k) if bf16 else k
     vf = oracle.bf16_to_f32(v) if bf16 else v
     ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
-    from moeflux_amd import ffi
+    s = q.reshape(Hq, d).astype(np.float64) @ kf.reshape(L, d).astype(np.float64).T / np.sqrt(d)
+    w = np.exp(s - s.max(axis=1, keepdims=True))
+    exact = ((w / w.sum(axis=1, keepdims=True)) @ vf.reshape(L, d).astype(np.float64)
+             / (1.0 + np.exp(-g.reshape(Hq, d).astype(np.float64)))).reshape(-1)
     with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
               head_dim=d, kv_capacity=L, kv_dtype=1 if bf16 else 0) as c:
         c.kv_import(0, kf, vf)
         base = c.sdpa_decode(0, q, g)
-        assert rel_err(base, ref) <= (1e-4 if bf16 else TOL_F32)
+        assert rel_err(base, exact) <= (1e-4 if bf16 else TOL_F32)
+        assert rel_err(base, ref) <= (1e-4 if bf16 else TOL_F32 + rel_err(ref, exact))
         seen = set()
         for ns in (300, 512, 1024):
             c.set_num_splits(ns)
             seen.add(c.lib.mfa_debug_num_splits(1 if bf16 else 0, Hq, Hkv, d, L, 256, ns))
             out = c.sdpa_decode(0, q, g)
-            assert rel_err(out, ref) <= (1e-4 if bf16 else TOL_F32), ns
+            assert rel_err(out, exact) <= (1e-4 if bf16 else TOL_F32), ns
             assert rel_err(out, base) <= 1e-5, ns
         assert max(seen) > 256
-
-
-@pytest.mark.parametrize("Hq,Hkv,d,L,bf16", [(32, 2, 256, 9000, True), (32, 2, 256, 3000, False),
-                                             (32, 4, 128, 4096, False), (16, 2, 128, 5000, True),
-                                             (8, 8, 64, 2500, False), (40, 2, 128, 3100, True)])
-def test_merge_inside_the_launch_equals_the_separate_launch(mfa, oracle, Hq, Hkv, d, L, bf16):
-    """The same partials combined by a second launch, by the workgroup that arrives last alone
-    (no helper waits), with the default helper wait and with a long one: bit-identical results,
-    at split counts that take the few-split path (3, 8, 12, 16), the many-split path with helpers
-    (17, 20, 40, 64, 130, 300) and the default plan; several calls in a row, so that both sets of
-    ticket records are used and cleared in turn."""
-    q, g, k, v = sdpa_random_inputs(900 + L, Hq, Hkv, d, L, bf16=bf16)
-    kf = oracle.bf16_to_f32(k) if bf16 else k
-    vf = oracle.bf16_to_f32(v) if bf16 else v
-    ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
-    with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
-              head_dim=d, kv_capacity=L, kv_dtype=1 if bf16 else 0) as c:
-        c.kv_import(0, kf, vf)
-        for ns in (0, 3, 8, 12, 16, 17, 20, 40, 64, 130, 300):
-            c.set_num_splits(ns)
-            c.set_merge(in_launch=False)
-            base = c.sdpa_decode(0, q, g)
-            assert rel_err(base, ref) <= (1e-4 if bf16 else TOL_F32), ns
-            for polls in (0, -1, 4000, 0, -1):
-                c.set_merge(in_launch=True, helper_polls=polls)
-                out = c.sdpa_decode(0, q, g)
-                assert np.array_equal(out, base), (ns, polls)
 
 
 def test_config3_full_size_bf16(mfa, oracle):

@@ -216,44 +216,6 @@ def test_stale_workspace_contents_never_reach_a_result(mfa, oracle, forced):
     assert rel_err_rows(out, ref, d) <= 3e-5
 
 
-def test_merge_inside_the_launch_for_chunks_and_sweeps(mfa, oracle):
-    """The merge run by the attention launch itself gives the bits of the merge as a second launch
-    where a launch has many row groups: a short chunk behind a long cache (per-row causal limits,
-    a ragged last row group, a split some rows cannot see), and the per-kind launch of a sweep
-    (all layers' kv heads in one grid); decode calls in between use the other set of ticket
-    records, whose used part each launch has to clear."""
-    from moeflux_amd import Config
-    from moeflux_amd.hip import DeviceArray
-    Hq, Hkv, d, T, L0 = 32, 2, 256, 21, 1020
-    rng = np.random.default_rng(5)
-    k = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
-    v = (rng.standard_normal((L0 + T, Hkv * d)) / np.sqrt(d)).astype(np.float32)
-    q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
-    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
-    ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
-    with _full_ctx(mfa, Hq, Hkv, d, L0 + T + 8, layers=3) as c:
-        outs = []
-        for mode in (False, True, True, False, True):
-            c.memory_clear()
-            for layer in range(3):
-                c.kv_import(layer, k[:L0], v[:L0])
-            c.set_merge(in_launch=mode)
-            o_chunk = c.prefill_attn(0, q, g, k[L0:], v[L0:])
-            o_dec = c.sdpa_decode(1, q[0], g[0])
-            # all three layers at once: layer 0 is T positions longer, so lengths differ -> per-layer loop;
-            # truncate it back to get the one-launch form
-            c.memory_seq_rm(L0)
-            dq, dg = DeviceArray.from_host(q[:3]), DeviceArray.from_host(g[:3])
-            do = DeviceArray((3, Hq * d), np.float32, zero=True)
-            assert c.lib.mfa_token_sweep_dev(c.h, dq.ptr, dg.ptr, do.ptr, None, None, None, None, None) == 0
-            c.sync()
-            outs.append((o_chunk, o_dec, do.to_host()))
-        assert rel_err(outs[0][0], ref) <= TOL_F32
-        for o in outs[1:]:
-            for a, b in zip(o, outs[0]):
-                assert np.array_equal(a, b)
-
-
 @pytest.mark.parametrize("per_layer", [0, 1])
 def test_config5_full_size_sweep(mfa, oracle, per_layer):
     """The 48-layer hybrid stack at its own size: layers 3, 7, ..., 47 full attention

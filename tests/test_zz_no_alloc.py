@@ -50,11 +50,11 @@ def test_static_scratch_decode_equals_the_workspace_decode(mfa, oracle, bf16):
 
 def test_static_scratch_refuses_a_plan_that_does_not_fit(mfa):
     """The automatic split plans stay within the array (a partial per workgroup, one or two
-    workgroups per CU); a forced count of 375 splits of 2 kv heads is 12 MiB of partial rows and
-    is refused with nothing launched."""
+    workgroups per CU); a forced count of 375 splits of 2 kv heads (the cache is long enough to give
+    each 64 positions) is 12 MiB of partial rows and is refused with nothing launched."""
     from moeflux_amd import Config, ffi
     from moeflux_amd.hip import DeviceArray
-    Hq, Hkv, d, L = 32, 2, 256, 12000
+    Hq, Hkv, d, L = 32, 2, 256, 24000
     cfg = Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
                  kv_capacity=L, kv_dtype=0)
     rng = np.random.default_rng(3)
@@ -64,8 +64,8 @@ def test_static_scratch_refuses_a_plan_that_does_not_fit(mfa):
         q = rng.standard_normal(Hq * d, dtype=np.float32)
         dq = DeviceArray.from_host(q)
         do = DeviceArray.from_host(np.full(q.shape, 7.0, np.float32))
-        c.set_num_splits(600)
-        assert c.lib.mfa_debug_num_splits(0, Hq, Hkv, d, L, 256, 600) * Hkv * 16 * d * 4 > 8 << 20
+        c.set_num_splits(375)
+        assert c.lib.mfa_debug_num_splits(0, Hq, Hkv, d, L, 256, 375) * Hkv * 16 * d * 4 > 8 << 20
         assert c.lib.mfa_sdpa_decode_static_dev(c.h, 0, dq.ptr, dq.ptr, do.ptr) == ffi.ERR_INVALID
         assert "static scratch" in ffi.last_error()
         c.sync()
