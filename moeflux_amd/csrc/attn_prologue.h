@@ -39,8 +39,7 @@ template <int LPH> __device__ inline float lanes_sum(float v) {
 template <int EPS, int D> struct HeadRotor {
     static constexpr int LPH = D / EPS;
     static_assert(LPH == 8 || LPH == 16 || LPH == 32 || LPH == 64, "a head's lanes fit a wave");
-    float cs[EPS], sn[EPS];
-    bool rot, low;
+    float cs[EPS], sn[EPS];   // cos, and sin with the sign of the lane's half: out = y cos + partner's y * sn
     int partner;
 
     // The workgroup's table of (cos, sin)(pos * inv_freq[i]), i < rotary_dim / 2, in LDS: thread i
@@ -53,17 +52,20 @@ template <int EPS, int D> struct HeadRotor {
     __device__ static inline void table(float freq, int pos, int rotary_dim, float2 *tab) {
         if ((int)threadIdx.x < (rotary_dim >> 1)) tab[threadIdx.x] = head_cos_sin((float)pos * freq);
     }
-    // j: the lane's index within its head
+    // j: the lane's index within its head.  The pair (x0, x1) = (channel c, channel c + half)
+    // becomes (x0 cos - x1 sin, x0 sin + x1 cos): the lane of the low channel holds y = x0 and gets
+    // x1 from its partner, the lane of the high channel holds y = x1 and gets x0, so both are
+    // y cos + other * (-sin | +sin); channels past rotary_dim have cos = 1, sin = 0 and themselves
+    // as partner.  No branch, and the lane exchanges of a slot are all issued before the first use.
     __device__ inline void init(int j, int rotary_dim, const float2 *tab) {
         const int c0 = EPS * j, half = rotary_dim >> 1;
-        rot = c0 < rotary_dim;
-        low = c0 < half;
+        const bool rot = c0 < rotary_dim, low = c0 < half;
 #pragma unroll
         for (int e = 0; e < EPS; e++) {
             const int c = c0 + e;
             const float2 t = tab[rot ? (c < half ? c : c - half) : 0];
             cs[e] = rot ? t.x : 1.f;
-            sn[e] = rot ? t.y : 0.f;
+            sn[e] = rot ? (low ? -t.y : t.y) : 0.f;
         }
         const int lane = threadIdx.x & 63, dj = half / EPS;
         partner = rot ? (low ? lane + dj : lane - dj) : lane;
@@ -75,13 +77,13 @@ template <int EPS, int D> struct HeadRotor {
         for (int e = 0; e < EPS; e++) ss += x[e] * x[e];
         ss = lanes_sum<LPH>(ss);
         const float inv_rms = 1.0f / sqrtf(ss / (float)D + eps);
+        float y[EPS], o[EPS];
 #pragma unroll
-        for (int e = 0; e < EPS; e++) {
-            const float y = x[e] * inv_rms * w[e];
-            const float o = __shfl(y, partner, 64);
-            const float x0 = low ? y : o, x1 = low ? o : y;
-            x[e] = !rot ? y : (low ? x0 * cs[e] - x1 * sn[e] : x0 * sn[e] + x1 * cs[e]);
-        }
+        for (int e = 0; e < EPS; e++) y[e] = x[e] * inv_rms * w[e];
+#pragma unroll
+        for (int e = 0; e < EPS; e++) o[e] = __shfl(y[e], partner, 64);
+#pragma unroll
+        for (int e = 0; e < EPS; e++) x[e] = y[e] * cs[e] + o[e] * sn[e];
     }
 };
 

@@ -167,16 +167,19 @@ __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_b
 // is fastest; the widest heads take sixteen, which also keeps the memory system busy while a
 // workgroup stages its query and exchanges its probabilities (bf16, head_dim 256, 32768 positions:
 // 13.2 us per launch with 8, 12.75 with 16, 12.9 with 32; 14.9 with 4).
-__host__ __device__ constexpr int ring_depth(bool bf16, int D) { return bf16 && D == 256 ? 16 : 8; }
+#ifndef MFA_STEP_RING
+#define MFA_STEP_RING 16
+#endif
+__host__ __device__ constexpr int ring_depth(bool bf16, int D, bool step = false) { return bf16 && D == 256 ? (step ? MFA_STEP_RING : 16) : 8; }
 
 // Shape constants of the streaming kernel.  A pass takes NCH chunks; its K is NCH * NK loads per
 // wave, its V as many.  The unified sequence of a wave's loads (K of a pass, its V, K of the next
 // pass, ...) runs through the ring with load number i in slot i % R, which holds as long as a pass
 // is at least one ring of K (MINCH chunks) and two of its phases are whole rings (chunk counts that
 // are multiples of GRAN): then every pass begins at slot 0 again.
-template <typename KV, int D> struct Stream {
+template <typename KV, int D, bool STEP = false> struct Stream {
     using W = Wave<KV, D>;
-    static constexpr int R = ring_depth(sizeof(KV) == 2, D);
+    static constexpr int R = ring_depth(sizeof(KV) == 2, D, STEP);
     static constexpr int CH = KvTile<KV>::KCH;              // positions of a K chunk
     static constexpr int NK = W::KSTEPS;                    // K loads per chunk and wave (one per k-step)
     static constexpr int VB = CH / W::BLK;                  // V blocks per chunk
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     int units_base, int units_rem, float qscale, float *__restrict__ part_o, float *__restrict__ part_ml,
     std::conditional_t<STEP, StepPrologue, NoPrologue> sp) {
     using W = Wave<KV, D>;
-    using S = Stream<KV, D>;
+    using S = Stream<KV, D, STEP>;
     constexpr int NK = S::NK, NV = S::NV, TPW = S::TPW, VB = S::VB, kRing = S::R;
     constexpr int NT = kWaves * 64;
     constexpr int NQ = (W::QSLOTS + NT - 1) / NT;  // query slots per thread
@@ -316,9 +319,20 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
         __builtin_amdgcn_sched_barrier(0);   // in ring order: loads return in the order of their requests
     }
 
+    // The rest of the ring follows when the first part has had time to arrive (a wave that asks for
+    // more than the CU's queue holds sits in the issue stage until data returns, and can do nothing
+    // else): in a decode step between the rotation table and the norms, which take as long again.
+    auto rest_of_ring = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = kHead; i < kRing; i++) {
+            ring[i] = k_load(c0 + i / NK, i % NK);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
     if constexpr (STEP) {
         HeadRotor<sq.EPS, D>::table(sq.freq, sp.pos, sp.rotary_dim, s_tab);
         lds_barrier();
+        rest_of_ring();
         sq.finish(sp, rows, qscale, plane_elems, with_new, qlds, nhg, s_tab);
     } else {
 #pragma unroll
@@ -326,11 +340,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
             const int slot = threadIdx.x + i * NT;
             if (slot < W::QSLOTS) W::store_q_slot(qlds, qraw[i], slot, qscale);
         }
-    }
-#pragma unroll
-    for (int i = kHead; i < kRing; i++) {
-        ring[i] = k_load(c0 + i / NK, i % NK);
-        __builtin_amdgcn_sched_barrier(0);
+        rest_of_ring();
     }
     lds_barrier();
     uint4 qr[W::QREGS];
@@ -541,15 +551,15 @@ bool sdpa_shape_supported(int kv_dtype, int head_dim) {
 }
 
 // chunks of a unit of the plan (Stream::GRAN)
-static int unit_chunks(int kv_dtype, int D) {
-    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
+static int unit_chunks(int kv_dtype, int D, bool step = false) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D, step);
     return (2 * nk) % ring == 0 ? 1 : ring / (2 * nk);
 }
 
 // chunks of the kernel's smallest pass (Stream::MINCH)
-static int min_pass_chunks(int kv_dtype, int D) {
-    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
-    const int m = (ring + nk - 1) / nk, g = unit_chunks(kv_dtype, D);
+static int min_pass_chunks(int kv_dtype, int D, bool step = false) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D, step);
+    const int m = (ring + nk - 1) / nk, g = unit_chunks(kv_dtype, D, step);
     return m < g ? g : m;
 }
 
@@ -578,12 +588,12 @@ static int64_t split_target(int Hq, int Hkv, int D, int64_t nhg, int64_t nunits,
 static constexpr int g_wgs_per_cu = 1;
 
 static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
-                             int num_cus, int forced) {
+                             int num_cus, int forced, bool step = false) {
     const int hpk = Hq / Hkv;
     SplitPlan p;
     p.nhg = (int)(((int64_t)n_tok * hpk + 15) / 16);
     const int64_t nchunk = (kv_len + kKvChunk - 1) / kKvChunk;
-    const int U = unit_chunks(kv_dtype, D);
+    const int U = unit_chunks(kv_dtype, D, step);
     int64_t nunits = (nchunk + U - 1) / U;
     if (nunits < 1) nunits = 1;
     int64_t target = forced > 0 ? forced : split_target(Hq, Hkv, D, p.nhg, nunits, num_cus, g_wgs_per_cu);
@@ -591,7 +601,7 @@ static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, in
     if (target > nunits) target = nunits;
     // a share smaller than the kernel's smallest pass would be padded with re-read chunks: the
     // automatic plan rather takes fewer workgroups
-    const int64_t min_units = (min_pass_chunks(kv_dtype, D) + U - 1) / U;
+    const int64_t min_units = (min_pass_chunks(kv_dtype, D, step) + U - 1) / U;
     if (forced <= 0 && target > 1 && nunits / target < min_units) target = nunits / min_units > 1 ? nunits / min_units : 1;
     p.splits = (int)target;
     p.base = (int)(nunits / target);
@@ -654,14 +664,14 @@ bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim) {
 // A plan that fits the workspace: an automatic split count shrinks to fit; one forced for a
 // single token is used as given or refused.
 static int fit_plan(SplitPlan &plan, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len, int num_cus,
-                    int forced_splits, const SdpaWorkspace &ws) {
+                    int forced_splits, const SdpaWorkspace &ws, bool step = false) {
     auto fits = [&](const SplitPlan &p) {
         return sdpa_workspace_o_elems(Hq, Hkv, D, p.splits, n_tok) <= ws.part_o_elems &&
                sdpa_workspace_ml_elems(Hq, Hkv, p.splits, n_tok) <= ws.part_ml_elems;
     };
-    plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
+    plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits, step);
     while ((forced_splits <= 0 || n_tok > 1) && plan.splits > 1 && !fits(plan))
-        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
+        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2, step);
     if (!fits(plan)) return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
     if (plan.nhg > 65535 || Hkv > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
     return MFA_OK;
@@ -681,7 +691,7 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
     if (len0 < 0 || pos < 0) return fail(MFA_ERR_INVALID, "attention step: negative position");
     const int hpk = Hq / Hkv;
     SplitPlan plan;
-    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits, ws));
+    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits, ws, true));
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     const StepPrologue sp{q_proj, k_in, v_in, q_norm, k_norm, inv_freq, rotary_dim, eps, pos, len0, new_score,
                           k_tiled, v_tiled, plan.splits - 1};
