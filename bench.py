@@ -32,10 +32,17 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the split-K partial kernel on the headline workload, from rocprofv3
-# FETCH_SIZE + WRITE_SIZE scaled by the plain copy kernel
-# (profiles/sdpa_partial_bf16_d256_c3_hbm_counters.md): 65 877 KiB read + 4 128 KiB written.
-C3_PARTIAL_TRAFFIC_BYTES = (65877 + 4128) * 1024
+
+
+def _c3_partial_traffic_bytes():
+    """HBM bytes per launch of the split-K partial kernel on the headline workload: rocprofv3
+    FETCH_SIZE + WRITE_SIZE scaled by the plain copy kernel, as recorded next to the counter summary
+    (profiles/sdpa_partial_bf16_d256_c3_hbm_counters.md); None when the record is missing."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "sdpa_partial_bf16_d256_c3_hbm_counters.json")) as f:
+            return int(json.load(f)["traffic_bytes_per_dispatch"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def _bf16_bits(x):
@@ -818,7 +825,7 @@ def main():
         "hbm_gbps": head["gbps"], "hbm_pct_peak": head["pct_peak"],
         "roofline": {"bound": "hbm", "achieved": head["gbps_partial_kernel"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": head["gbps_partial_kernel"] / HBM_PEAK_GBPS,
-                     "traffic": C3_PARTIAL_TRAFFIC_BYTES, "kernel": "sdpa_partial_kernel<bf16, 256, 8>",
+                     "traffic": _c3_partial_traffic_bytes(), "kernel": "sdpa_partial_kernel<bf16, 256>",
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
                      "us_per_launch": head["us_partial_kernel_loop"]},
     }
