@@ -7,14 +7,17 @@
 // sdpa_cpu (crates/moeflux/src/riir/sdpa.rs:63-172) with two launches:
 //
 //   sdpa_partial_kernel  grid (splits, 16-row groups, kv heads), 4 waves.
-//     A workgroup streams its share of the cache: K and V pass through a ring of eight 1 KiB
-//     loads per wave, each consumed by the matrix core as it arrives and replaced by the next
-//     request, so a CU keeps 32 KiB in flight and its four waves, reading side by side, sweep
+//     A workgroup streams its share of the cache: K and V pass through a ring of 1 KiB loads
+//     per wave (16 for bf16 caches of head_dim 256, else 8), each consumed by the matrix core as
+//     it arrives and replaced by the next request, so a CU keeps 32-64 KiB in flight and its
+//     four waves, reading side by side, sweep
 //     one contiguous run of memory (measured on 64 MiB: 10.8 us per launch in this pattern,
 //     12.8 us with a workgroup's whole share requested at once, 11.5-12 us with one contiguous
 //     run per wave).  The up to 16 query heads that share the kv head are the N dimension of the
 //     matrix instruction, so lane % 16 is the head index throughout.  The cache is consumed in
-//     passes of up to G chunks of 64 positions:
+//     passes of whole chunks of 64 positions; the chunk count of a pass is a compile-time
+//     constant (so ring slots are registers), the main loop takes passes of 4 (f32: 2) chunks and
+//     the tail one pass of whatever is left, chosen among the compiled forms:
 //       K phase  wave w owns the 16-position sub-tile w of every chunk:
 //                S^T[pos, head] += K[pos, k-step] . Q[head, k-step] per load, the query operands
 //                in registers; while the last K loads are consumed the first V loads go out.
@@ -167,10 +170,7 @@ __device__ inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_b
 // is fastest; the widest heads take sixteen, which also keeps the memory system busy while a
 // workgroup stages its query and exchanges its probabilities (bf16, head_dim 256, 32768 positions:
 // 13.2 us per launch with 8, 12.75 with 16, 12.9 with 32; 14.9 with 4).
-#ifndef MFA_STEP_RING
-#define MFA_STEP_RING 16
-#endif
-__host__ __device__ constexpr int ring_depth(bool bf16, int D, bool step = false) { return bf16 && D == 256 ? (step ? MFA_STEP_RING : 16) : 8; }
+__host__ __device__ constexpr int ring_depth(bool bf16, int D) { return bf16 && D == 256 ? 16 : 8; }
 
 // Shape constants of the streaming kernel.  A pass takes NCH chunks; its K is NCH * NK loads per
 // wave, its V as many.  The unified sequence of a wave's loads (K of a pass, its V, K of the next
@@ -179,7 +179,7 @@ __host__ __device__ constexpr int ring_depth(bool bf16, int D, bool step = false
 // are multiples of GRAN): then every pass begins at slot 0 again.
 template <typename KV, int D, bool STEP = false> struct Stream {
     using W = Wave<KV, D>;
-    static constexpr int R = ring_depth(sizeof(KV) == 2, D, STEP);
+    static constexpr int R = ring_depth(sizeof(KV) == 2, D);
     static constexpr int CH = KvTile<KV>::KCH;              // positions of a K chunk
     static constexpr int NK = W::KSTEPS;                    // K loads per chunk and wave (one per k-step)
     static constexpr int VB = CH / W::BLK;                  // V blocks per chunk
@@ -551,15 +551,15 @@ bool sdpa_shape_supported(int kv_dtype, int head_dim) {
 }
 
 // chunks of a unit of the plan (Stream::GRAN)
-static int unit_chunks(int kv_dtype, int D, bool step = false) {
-    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D, step);
+static int unit_chunks(int kv_dtype, int D) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
     return (2 * nk) % ring == 0 ? 1 : ring / (2 * nk);
 }
 
 // chunks of the kernel's smallest pass (Stream::MINCH)
-static int min_pass_chunks(int kv_dtype, int D, bool step = false) {
-    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D, step);
-    const int m = (ring + nk - 1) / nk, g = unit_chunks(kv_dtype, D, step);
+static int min_pass_chunks(int kv_dtype, int D) {
+    const int nk = kv_dtype == MFA_KV_BF16 ? D / 32 : D / 16, ring = ring_depth(kv_dtype == MFA_KV_BF16, D);
+    const int m = (ring + nk - 1) / nk, g = unit_chunks(kv_dtype, D);
     return m < g ? g : m;
 }
 
@@ -588,12 +588,12 @@ static int64_t split_target(int Hq, int Hkv, int D, int64_t nhg, int64_t nunits,
 static constexpr int g_wgs_per_cu = 1;
 
 static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
-                             int num_cus, int forced, bool step = false) {
+                             int num_cus, int forced) {
     const int hpk = Hq / Hkv;
     SplitPlan p;
     p.nhg = (int)(((int64_t)n_tok * hpk + 15) / 16);
     const int64_t nchunk = (kv_len + kKvChunk - 1) / kKvChunk;
-    const int U = unit_chunks(kv_dtype, D, step);
+    const int U = unit_chunks(kv_dtype, D);
     int64_t nunits = (nchunk + U - 1) / U;
     if (nunits < 1) nunits = 1;
     int64_t target = forced > 0 ? forced : split_target(Hq, Hkv, D, p.nhg, nunits, num_cus, g_wgs_per_cu);
@@ -601,7 +601,7 @@ static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, in
     if (target > nunits) target = nunits;
     // a share smaller than the kernel's smallest pass would be padded with re-read chunks: the
     // automatic plan rather takes fewer workgroups
-    const int64_t min_units = (min_pass_chunks(kv_dtype, D, step) + U - 1) / U;
+    const int64_t min_units = (min_pass_chunks(kv_dtype, D) + U - 1) / U;
     if (forced <= 0 && target > 1 && nunits / target < min_units) target = nunits / min_units > 1 ? nunits / min_units : 1;
     p.splits = (int)target;
     p.base = (int)(nunits / target);
@@ -664,14 +664,14 @@ bool sdpa_step_supported(int kv_dtype, int Hq, int Hkv, int D, int rotary_dim) {
 // A plan that fits the workspace: an automatic split count shrinks to fit; one forced for a
 // single token is used as given or refused.
 static int fit_plan(SplitPlan &plan, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len, int num_cus,
-                    int forced_splits, const SdpaWorkspace &ws, bool step = false) {
+                    int forced_splits, const SdpaWorkspace &ws) {
     auto fits = [&](const SplitPlan &p) {
         return sdpa_workspace_o_elems(Hq, Hkv, D, p.splits, n_tok) <= ws.part_o_elems &&
                sdpa_workspace_ml_elems(Hq, Hkv, p.splits, n_tok) <= ws.part_ml_elems;
     };
-    plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits, step);
+    plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, forced_splits);
     while ((forced_splits <= 0 || n_tok > 1) && plan.splits > 1 && !fits(plan))
-        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2, step);
+        plan = plan_splits(kv_dtype, Hq, Hkv, D, n_tok, kv_len, num_cus, (plan.splits + 1) / 2);
     if (!fits(plan)) return fail(MFA_ERR_INVALID, "sdpa: split-K workspace too small for %d splits", plan.splits);
     if (plan.nhg > 65535 || Hkv > 65535) return fail(MFA_ERR_SHAPE, "sdpa: too many query rows in one call");
     return MFA_OK;
@@ -691,7 +691,7 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
     if (len0 < 0 || pos < 0) return fail(MFA_ERR_INVALID, "attention step: negative position");
     const int hpk = Hq / Hkv;
     SplitPlan plan;
-    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits, ws, true));
+    MFA_TRY(fit_plan(plan, kv_dtype, Hq, Hkv, D, 1, len0 > 0 ? len0 : 1, num_cus, forced_splits, ws));
     const float qscale = (1.0f / sqrtf((float)D)) * kLog2e;
     const StepPrologue sp{q_proj, k_in, v_in, q_norm, k_norm, inv_freq, rotary_dim, eps, pos, len0, new_score,
                           k_tiled, v_tiled, plan.splits - 1};
