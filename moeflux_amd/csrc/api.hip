@@ -60,6 +60,16 @@ int ensure_stage(Ctx *c, size_t elems) {
     return MFA_OK;
 }
 
+int release_stage_beyond_cap(Ctx *c) {
+    if (c->stage_elems <= kStageCap) return MFA_OK;
+    MFA_HIP(hipFree(c->stage));
+    c->stage = nullptr;
+    c->stage_elems = 0;
+    // (hipMemGetInfo shows the bytes again once another command has followed the stream's last one:
+    // the runtime keeps a freed buffer alive as long as the last command submitted refers to it)
+    return MFA_OK;
+}
+
 static SdpaWorkspace workspace(Ctx *c) {
     return SdpaWorkspace{c->part_o, c->part_ml, c->part_o_elems, c->part_ml_elems};
 }
@@ -1067,7 +1077,8 @@ int mfa_kv_export(mfa_ctx *ctx, int32_t layer, int32_t max_rows, float *k_out, f
     MFA_TRY(launch_kv_gather(c->stream, c->cfg.kv_dtype, c->cfg.num_kv_heads, c->cfg.head_dim,
                              c->plane_elems, f->len, f->k, f->v, c->stage, c->stage + n));
     MFA_HIP(hipMemcpyAsync(k_out, c->stage, n * 4, hipMemcpyDeviceToHost, c->stream));
-    return d2h_sync(c, v_out, c->stage + n, n * 4);
+    MFA_TRY(d2h_sync(c, v_out, c->stage + n, n * 4));
+    return release_stage_beyond_cap(c);
 }
 
 
@@ -1111,7 +1122,7 @@ static int kv_import(Ctx *c, int32_t layer, int32_t len, const void *k, const vo
     }
     f->len = len;
     MFA_HIP(hipStreamSynchronize(c->stream));
-    return MFA_OK;
+    return release_stage_beyond_cap(c);
 }
 
 int mfa_kv_import(mfa_ctx *ctx, int32_t layer, int32_t len, const float *k, const float *v) {

@@ -193,6 +193,11 @@ inline Ctx *as_ctx(mfa_ctx *c) { return reinterpret_cast<Ctx *>(c); }
 int full_layer(Ctx *c, int32_t layer, FullLayer **out);
 int linear_layer(Ctx *c, int32_t layer, LinearLayer **out);
 int ensure_stage(Ctx *c, size_t elems);
+// The staging buffer a context keeps between calls is at most this many floats (256 MiB): the bulk
+// entry points (snapshot, cache import and export), whose staging grows with the cache length, call
+// release_stage_beyond_cap once their work on the stream has completed.
+static constexpr size_t kStageCap = ((size_t)256 << 20) / sizeof(float);
+int release_stage_beyond_cap(Ctx *c);
 // api.hip: device-to-device halves of the state export and import calls (no synchronisation)
 int kv_export_to(Ctx *c, FullLayer *f, float *k_dev, float *v_dev);
 int kv_import_from(Ctx *c, FullLayer *f, int32_t len, const float *k_dev, const float *v_dev);

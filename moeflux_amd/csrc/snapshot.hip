@@ -11,6 +11,7 @@
 // Saved as version 2 (what the reference writes); versions 1 and 2 load.  A bf16 cache is
 // widened on save and rounded back on load, which is exact for values that were bf16.
 #include <cstring>
+#include <vector>
 
 #include "mfa_internal.h"
 
@@ -42,6 +43,27 @@ static uint32_t get_u32(const uint8_t *p) {
 static constexpr size_t kSegAlign = 64;
 static size_t seg_round(size_t elems) { return (elems + kSegAlign - 1) / kSegAlign * kSegAlign; }
 
+// The image is built for runs of consecutive layers whose segments fit kStageCap together (a layer
+// larger than that is a run of its own), so the staging buffer a snapshot needs does not grow with
+// the number of layers; the runs follow one another on the stream and reuse the buffer in stream
+// order.  What a long cache made the buffer grow beyond the cap is given back when the call ends
+// (release_stage_beyond_cap).
+
+// seg[i]: image elements of layer i.  Returns the ends of the runs and the largest run.
+static std::vector<int> layer_runs(const std::vector<size_t> &seg, size_t *largest) {
+    std::vector<int> ends;
+    *largest = 0;
+    for (size_t i = 0; i < seg.size();) {
+        size_t img = seg[i], j = i + 1;
+        while (j < seg.size() && img + seg[j] <= kStageCap) img += seg[j++];
+        if (img > *largest) *largest = img;
+        ends.push_back((int)j);
+        i = j;
+    }
+    return ends;
+}
+
+
 }  // namespace mfa
 
 using namespace mfa;
@@ -67,41 +89,46 @@ int64_t mfa_state_save(mfa_ctx *ctx, uint8_t *buf, int64_t buf_len) {
     const uint32_t header[kHeaderV2] = {kMagic, kVersion, (uint32_t)c->cfg.num_layers, (uint32_t)c->cfg.full_attn_interval,
                                         (uint32_t)c->cfg.num_kv_heads, (uint32_t)c->cfg.head_dim,
                                         (uint32_t)conv_bytes(c), (uint32_t)ssm_bytes(c), 0u, 0u};
-    // every layer's rows are gathered into the device image first, then the copies follow one
-    // another on the stream, and the host waits once
-    size_t img = 0;
+    // a run's rows are gathered into the device image first, then its copies follow one another on
+    // the stream; the host waits once, after the last run
+    std::vector<size_t> seg(c->cfg.num_layers);
     for (int i = 0; i < c->cfg.num_layers; i++)
-        img += c->kind[i] == 1 ? seg_round(2 * (size_t)c->full[c->slot[i]].len * c->kv_dim()) : seg_round(conv_bytes(c) / 4);
-    MFA_TRY(ensure_stage(c, img));
-    size_t at = 0;
-    for (int i = 0; i < c->cfg.num_layers; i++) {
-        if (c->kind[i] == 1) {
-            FullLayer *f = &c->full[c->slot[i]];
-            const size_t n = (size_t)f->len * c->kv_dim();
-            MFA_TRY(kv_export_to(c, f, c->stage + at, c->stage + at + n));
-            at += seg_round(2 * n);
-        } else {
-            MFA_TRY(linear_export_to(c, &c->lin[c->slot[i]], c->stage + at));
-            at += seg_round(conv_bytes(c) / 4);
-        }
-    }
+        seg[i] = c->kind[i] == 1 ? seg_round(2 * (size_t)c->full[c->slot[i]].len * c->kv_dim()) : seg_round(conv_bytes(c) / 4);
+    size_t largest = 0;
+    const std::vector<int> runs = layer_runs(seg, &largest);
+    MFA_TRY(ensure_stage(c, largest));
     size_t off = kHeaderV2 * 4;
-    at = 0;
-    for (int i = 0; i < c->cfg.num_layers; i++) {
-        if (c->kind[i] == 1) {
-            const size_t n = (size_t)c->full[c->slot[i]].len * c->kv_dim();
-            off += 4;
-            if (n > 0) MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, 2 * n * 4, hipMemcpyDeviceToHost, c->stream));
-            off += 2 * n * 4;
-            at += seg_round(2 * n);
-        } else {
-            MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, conv_bytes(c), hipMemcpyDeviceToHost, c->stream));
-            MFA_HIP(hipMemcpyAsync(buf + off + conv_bytes(c), c->lin[c->slot[i]].ssm, ssm_bytes(c), hipMemcpyDeviceToHost, c->stream));
-            off += conv_bytes(c) + ssm_bytes(c);
-            at += seg_round(conv_bytes(c) / 4);
+    int first = 0;
+    for (int end : runs) {
+        size_t at = 0;
+        for (int i = first; i < end; i++) {
+            if (c->kind[i] == 1) {
+                FullLayer *f = &c->full[c->slot[i]];
+                const size_t n = (size_t)f->len * c->kv_dim();
+                MFA_TRY(kv_export_to(c, f, c->stage + at, c->stage + at + n));
+            } else {
+                MFA_TRY(linear_export_to(c, &c->lin[c->slot[i]], c->stage + at));
+            }
+            at += seg[i];
         }
+        at = 0;
+        for (int i = first; i < end; i++) {
+            if (c->kind[i] == 1) {
+                const size_t n = (size_t)c->full[c->slot[i]].len * c->kv_dim();
+                off += 4;
+                if (n > 0) MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, 2 * n * 4, hipMemcpyDeviceToHost, c->stream));
+                off += 2 * n * 4;
+            } else {
+                MFA_HIP(hipMemcpyAsync(buf + off, c->stage + at, conv_bytes(c), hipMemcpyDeviceToHost, c->stream));
+                MFA_HIP(hipMemcpyAsync(buf + off + conv_bytes(c), c->lin[c->slot[i]].ssm, ssm_bytes(c), hipMemcpyDeviceToHost, c->stream));
+                off += conv_bytes(c) + ssm_bytes(c);
+            }
+            at += seg[i];
+        }
+        first = end;
     }
     MFA_HIP(hipStreamSynchronize(c->stream));
+    MFA_TRY(release_stage_beyond_cap(c));
     // the words the host knows: header and cache lengths
     off = 0;
     for (uint32_t w : header) { put_u32(buf + off, w); off += 4; }
@@ -168,40 +195,46 @@ int mfa_state_load(mfa_ctx *ctx, const uint8_t *buf, int64_t buf_len) {
             q += bytes;
         }
     }
-    // restore: every layer's bytes go to the device image first (a copy from pageable memory has
-    // left the caller's buffer when the call returns), then the kernels unpack them; one wait
-    size_t img = 0, off = header_bytes;
+    // restore: a run's bytes go to the device image first (a copy from pageable memory has left the
+    // caller's buffer when the call returns), then the kernels unpack them; one wait at the end
+    std::vector<size_t> seg(c->cfg.num_layers);
+    size_t off = header_bytes;
     for (int i = 0; i < c->cfg.num_layers; i++) {
         if (c->kind[i] == 1) {
             const int32_t len = (int32_t)get_u32(buf + off);
             off += 4 + 2 * (size_t)len * row_bytes(c);
-            img += seg_round(2 * (size_t)len * c->kv_dim());
+            seg[i] = seg_round(2 * (size_t)len * c->kv_dim());
         } else {
             off += conv_bytes(c) + ssm_bytes(c);
-            img += seg_round(conv_bytes(c) / 4);
+            seg[i] = seg_round(conv_bytes(c) / 4);
         }
     }
-    MFA_TRY(ensure_stage(c, img));
+    size_t largest = 0;
+    const std::vector<int> runs = layer_runs(seg, &largest);
+    MFA_TRY(ensure_stage(c, largest));
     off = header_bytes;
-    size_t at = 0;
-    for (int i = 0; i < c->cfg.num_layers; i++) {
-        if (c->kind[i] == 1) {
-            const int32_t len = (int32_t)get_u32(buf + off);
-            off += 4;
-            const size_t n = (size_t)len * c->kv_dim();
-            if (n > 0) MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, 2 * n * 4, hipMemcpyHostToDevice, c->stream));
-            MFA_TRY(kv_import_from(c, &c->full[c->slot[i]], len, c->stage + at, c->stage + at + n));
-            off += 2 * n * 4;
-            at += seg_round(2 * n);
-        } else {
-            LinearLayer *l = &c->lin[c->slot[i]];
-            MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, conv_bytes(c), hipMemcpyHostToDevice, c->stream));
-            MFA_TRY(linear_import_from(c, l, c->stage + at));
-            MFA_HIP(hipMemcpyAsync(l->ssm, buf + off + conv_bytes(c), ssm_bytes(c), hipMemcpyHostToDevice, c->stream));
-            off += conv_bytes(c) + ssm_bytes(c);
-            at += seg_round(conv_bytes(c) / 4);
+    int first = 0;
+    for (int end : runs) {
+        size_t at = 0;
+        for (int i = first; i < end; i++) {
+            if (c->kind[i] == 1) {
+                const int32_t len = (int32_t)get_u32(buf + off);
+                off += 4;
+                const size_t n = (size_t)len * c->kv_dim();
+                if (n > 0) MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, 2 * n * 4, hipMemcpyHostToDevice, c->stream));
+                MFA_TRY(kv_import_from(c, &c->full[c->slot[i]], len, c->stage + at, c->stage + at + n));
+                off += 2 * n * 4;
+            } else {
+                LinearLayer *l = &c->lin[c->slot[i]];
+                MFA_HIP(hipMemcpyAsync(c->stage + at, buf + off, conv_bytes(c), hipMemcpyHostToDevice, c->stream));
+                MFA_TRY(linear_import_from(c, l, c->stage + at));
+                MFA_HIP(hipMemcpyAsync(l->ssm, buf + off + conv_bytes(c), ssm_bytes(c), hipMemcpyHostToDevice, c->stream));
+                off += conv_bytes(c) + ssm_bytes(c);
+            }
+            at += seg[i];
         }
+        first = end;
     }
     MFA_HIP(hipStreamSynchronize(c->stream));
-    return MFA_OK;
+    return release_stage_beyond_cap(c);
 }

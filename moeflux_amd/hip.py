@@ -26,6 +26,7 @@ def rt() -> C.CDLL:
         _rt.hipGetErrorString.restype = C.c_char_p
         _rt.hipGetErrorString.argtypes = [C.c_int]
         _rt.hipGetDeviceCount.argtypes = [C.POINTER(C.c_int)]
+        _rt.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
     return _rt
 
 
@@ -38,6 +39,13 @@ def device_count() -> int:
     n = C.c_int(0)
     rc = rt().hipGetDeviceCount(C.byref(n))
     return n.value if rc == 0 else 0
+
+
+def mem_free() -> int:
+    """Free device memory in bytes (hipMemGetInfo) on the current device."""
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    _check(rt().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value
 
 
 def synchronize() -> None:

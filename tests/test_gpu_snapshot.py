@@ -141,3 +141,50 @@ def test_snapshot_rejections_leave_the_context_untouched(mfa, oracle):
             assert c.state_save() == before, name
         c.state_load(blob)
         assert c.state_save() == blob
+
+
+def test_snapshot_larger_than_the_staging_buffer(mfa, oracle):
+    """The device image of a snapshot is built in runs of layers of at most 256 MiB (a larger layer
+    alone), so the staging memory does not grow with the state: four full-attention layers of
+    82/164/328/41 MiB with linear layers between them (runs of three layers, an oversize layer alone,
+    the rest) give the bytes the per-layer exports give, load back to the same bytes, and once the
+    oversize run's buffer is released the calls hold no more than the 256 MiB they may keep."""
+    from moeflux_amd import Config
+    from moeflux_amd.hip import mem_free
+    hkv, d = 2, 256
+    lens = {1: 21000, 3: 42000, 5: 84000, 7: 10500}
+    cfg = Config(num_layers=8, full_attn_interval=2, num_attn_heads=8, num_kv_heads=hkv, head_dim=d,
+                 kv_capacity=84032, kv_dtype=1, linear_num_k_heads=2, linear_num_v_heads=4,
+                 linear_key_dim=64, linear_value_dim=64)
+    case = GdnCase(3, 2, 4, 64, 64, T=2)
+    rng = np.random.default_rng(5)
+    with mfa.Ctx(cfg) as c:
+        for layer, n in lens.items():
+            k = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal((n, hkv * d), dtype=np.float32)))
+            c.kv_import(layer, k, k[::-1].copy())
+        for layer in (0, 2, 4, 6):
+            c.set_linear_weights(layer, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
+            c.linear_state_import(layer, case.conv_state * (layer + 1), case.ssm_state)
+        probe = rng.standard_normal(8 * d, dtype=np.float32)
+        c.sdpa_decode(7, probe, probe)
+        free0 = mem_free()
+        blob = c.state_save()
+        c.sdpa_decode(7, probe, probe)
+        assert mem_free() >= free0 - (8 << 20)
+        want = bytearray(blob[:40])
+        for layer in range(8):
+            if layer in lens:
+                k, v = c.kv_export(layer)
+                want += struct.pack("<i", k.shape[0]) + k.tobytes() + v.tobytes()
+            else:
+                cs, ss = c.linear_state_export(layer)
+                want += cs.astype("<f4").tobytes() + ss.astype("<f4").tobytes()
+        assert bytes(want) == blob
+        del want
+        c.memory_clear()
+        c.state_load(blob)
+        assert [c.kv_len(layer) for layer in (1, 3, 5, 7)] == [21000, 42000, 84000, 10500]
+        # the runtime returns a freed buffer once another command has followed the last one that used it
+        c.sdpa_decode(7, probe, probe)
+        assert mem_free() >= free0 - (256 << 20) - (8 << 20)
+        assert c.state_save() == blob

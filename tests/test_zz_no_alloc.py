@@ -48,6 +48,37 @@ def test_static_scratch_decode_equals_the_workspace_decode(mfa, oracle, bf16):
         assert np.array_equal(ws, st)
 
 
+def test_static_scratch_decode_leaves_the_free_device_memory_as_it_was(mfa):
+    """What the entry point is for: no allocation.  Free device memory (hipMemGetInfo) is read before
+    and after calls over cache lengths that change the split plan from 1 workgroup per row group to
+    128 and back; not a byte may have moved, where the same sweep through a fresh context's first
+    ordinary decode may grow its workspace."""
+    from moeflux_amd import Config, ffi
+    from moeflux_amd.hip import DeviceArray, mem_free
+    Hq, Hkv, d, L = 32, 2, 256, 33000
+    cfg = Config(num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                 kv_capacity=L, kv_dtype=1)
+    rng = np.random.default_rng(8)
+    k = rng.standard_normal((L, Hkv * d), dtype=np.float32)
+    q = rng.standard_normal(Hq * d, dtype=np.float32)
+    with mfa.Ctx(cfg) as c:
+        c.kv_import(0, k, k[::-1].copy())
+        dq = DeviceArray.from_host(q)
+        do = DeviceArray.from_host(np.zeros(q.shape, np.float32))
+        c.sync()
+        plans = set()
+        free0 = mem_free()
+        for n in (33000, 8192, 700, 64, 1):
+            c.memory_seq_rm(n)
+            assert c.kv_len(0) == n
+            plans.add(c.lib.mfa_debug_num_splits(1, Hq, Hkv, d, n, 256, 0))
+            assert c.lib.mfa_sdpa_decode_static_dev(c.h, 0, dq.ptr, dq.ptr, do.ptr) == 0, ffi.last_error()
+            c.sync()
+            assert mem_free() == free0, n
+        assert len(plans) >= 3 and max(plans) >= 64 and min(plans) == 1
+        assert np.isfinite(do.to_host()).all()
+
+
 def test_static_scratch_refuses_a_plan_that_does_not_fit(mfa):
     """The automatic split plans stay within the array (a partial per workgroup, one or two
     workgroups per CU); a forced count of 375 splits of 2 kv heads (the cache is long enough to give
