@@ -187,6 +187,9 @@ template <typename KV, int D, bool STEP = false> struct Stream {
     static constexpr int NV = VB * TPW;                     // V loads per chunk and wave
     static constexpr int GRAN = (2 * NK) % R == 0 ? 1 : R / (2 * NK);   // chunk counts of a pass are multiples of this
     static constexpr int MINCH = (R + NK - 1) / NK < GRAN ? GRAN : (R + NK - 1) / NK;   // chunks of the smallest pass
+    // A share of a single unit is less than a ring of K where MINCH > GRAN; then its K and V together
+    // are exactly one ring, requested whole before the query is staged (the short form).
+    static constexpr bool HAS_SHORT = MINCH > GRAN;
     // A workgroup's share is streamed in passes of MAIN chunks until at most GMAX are left, which
     // are one last pass: one exchange of maxima and probabilities per pass, and a share a little
     // larger than the others' (a cache just past a multiple of the workgroups' shares) still is
@@ -196,6 +199,7 @@ template <typename KV, int D, bool STEP = false> struct Stream {
     static constexpr int KCH_U4 = CH * D * (int)sizeof(KV) / 16;      // 16-byte words of a chunk of K
     static constexpr int VBLK_U4 = W::BLK * D * (int)sizeof(KV) / 16;  // of a block of V
     static_assert(NV == NK && W::NACC % kWaves == 0, "K and V of a chunk are the same number of loads");
+    static_assert(!HAS_SHORT || 2 * GRAN * NK == R, "the short form fills the ring exactly");
     static_assert(MAIN % GRAN == 0 && GMAX % GRAN == 0 && MAIN >= MINCH && GMAX - MAIN + GRAN >= MINCH,
                   "every pass of a long share is a whole form");
 };
@@ -313,9 +317,22 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     };
     uint4 ring[kRing];
     constexpr int kHead = kRing < 8 ? kRing : 8;   // of the ring's first requests, those made before the query is staged
+    // The ring's first filling is the first kRing loads of the share's sequence: K of its first
+    // chunks, or, for a share of one unit where that is half a ring, its K and then its V.
+    const bool short_share = S::HAS_SHORT && c1 - c0 <= S::GRAN;
+    auto first_load = [&](int i) __attribute__((always_inline)) {
+        constexpr int KS = S::GRAN * NK;   // K loads of the short form
+        if (S::HAS_SHORT && i >= KS) {
+            const int64_t kc = (c0 + i / NK < cmax ? c0 + i / NK : cmax) * S::KCH_U4 + (i % NK) * 256;
+            const int64_t vb0 = c0 * VB + (i - KS) / TPW;
+            const int64_t vc = (vb0 < vmax ? vb0 : vmax) * S::VBLK_U4 + ((i - KS) % TPW) * 256;
+            return stream_load(short_share ? vbase + vc : kbase + kc);
+        }
+        return k_load(c0 + i / NK, i % NK);
+    };
 #pragma unroll
     for (int i = 0; i < kHead; i++) {
-        ring[i] = k_load(c0 + i / NK, i % NK);
+        ring[i] = first_load(i);
         __builtin_amdgcn_sched_barrier(0);   // in ring order: loads return in the order of their requests
     }
 
@@ -325,7 +342,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     auto rest_of_ring = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = kHead; i < kRing; i++) {
-            ring[i] = k_load(c0 + i / NK, i % NK);
+            ring[i] = first_load(i);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -360,7 +377,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
         constexpr bool MORE = decltype(more_tag)::value;
         constexpr int KL = NCH * NK, VL = NCH * NV;
         constexpr int VO = KL % kRing;   // ring slot of the pass's first V load
-        static_assert(KL >= kRing && (KL + VL) % kRing == 0, "a ring of K at least, and the next pass begins at slot 0");
+        static_assert((KL + VL) % kRing == 0 && (KL >= kRing || (!MORE && KL + VL == kRing)),
+                      "a ring of K at least and the next pass begins at slot 0, or the whole share in one ring");
         // ---- K phase: this wave's sub-tile of every chunk ----------------------------------
         f32x4 sc[NCH];
 #pragma unroll
@@ -369,7 +387,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
         for (int i = 0; i < KL; i++) {
             sc[i / NK] = W::score_step(ring[i % kRing], qr, i % NK, sc[i / NK]);
             if (i + kRing < KL) ring[i % kRing] = k_load(cb + (i + kRing) / NK, (i + kRing) % NK);
-            else ring[i % kRing] = v_load(cb * VB + (i + kRing - KL) / TPW, (i + kRing - KL) % TPW);
+            else if (i + kRing - KL < VL) ring[i % kRing] = v_load(cb * VB + (i + kRing - KL) / TPW, (i + kRing - KL) % TPW);
             // the request stays here, a ring's length ahead of its use (left alone the scheduler
             // sinks it to just before the use, and the ring runs one or two deep)
             __builtin_amdgcn_sched_barrier(0);
@@ -439,7 +457,11 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     for (; c1 - cb > S::GMAX; cb += S::MAIN) pass(cb, std::integral_constant<int, S::MAIN>{}, std::true_type{});
     // the last pass, in the smallest form that holds what is left (a form's chunks past the split's
     // end re-read its last chunk and are masked)
-    with_form<S::MINCH, S::GMAX, S::GRAN>((int)(c1 - cb), [&](auto nch) __attribute__((always_inline)) { pass(cb, nch, std::false_type{}); });
+    if (short_share) {
+        if constexpr (S::HAS_SHORT) pass(cb, std::integral_constant<int, S::GRAN>{}, std::false_type{});
+    } else {
+        with_form<S::MINCH, S::GMAX, S::GRAN>((int)(c1 - cb), [&](auto nch) __attribute__((always_inline)) { pass(cb, nch, std::false_type{}); });
+    }
 
     // ---- one partial per workgroup -----------------------------------------------
     l_run += lane_xor(l_run, 16);
@@ -599,8 +621,9 @@ static SplitPlan plan_splits(int kv_dtype, int Hq, int Hkv, int D, int n_tok, in
     int64_t target = forced > 0 ? forced : split_target(Hq, Hkv, D, p.nhg, nunits, num_cus, g_wgs_per_cu);
     if (target > kMaxSplits) target = kMaxSplits;
     if (target > nunits) target = nunits;
-    // a share smaller than the kernel's smallest pass would be padded with re-read chunks: the
-    // automatic plan rather takes fewer workgroups
+    // the automatic plan keeps a share at least the kernel's smallest pass of whole rings: shares of a
+    // single unit (the short form) on twice the workgroups measured slower (12 layers of 8192
+    // positions, head_dim 256, bf16: 128 x 1 chunk against 64 x 2 chunks, +0.5 us per layer)
     const int64_t min_units = (min_pass_chunks(kv_dtype, D) + U - 1) / U;
     if (forced <= 0 && target > 1 && nunits / target < min_units) target = nunits / min_units > 1 ? nunits / min_units : 1;
     p.splits = (int)target;
