@@ -51,6 +51,11 @@ def _bf16_bits(x):
     return ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
 
 
+def _bf16_round(x):
+    """f32 values rounded to the nearest bf16, as f32."""
+    return (_bf16_bits(x).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
 class _GdnInputs:
     """Synthetic constants, state and T tokens of inputs of one Gated-DeltaNet layer at the step
     shape the metric names: A_log = 0, dt_bias = 0, norm weight 1, conv weights ~ N(0, 0.5) in bf16."""
@@ -232,6 +237,17 @@ def bench_prefill(steps, warmup, seed, T=512):
            "attention_tflops": flops / (ev_ms * 1e-3) / 1e12,
            "attention_us_per_token_layer": ev_ms * 1e3 / T}
     ctx.close()
+    # The same chunk with a query that is exact in bf16 (what a bf16 model hands over, and what
+    # the configuration's "bf16" says): its low parts are zero and the kernel leaves their products out.
+    dqb = DeviceArray.from_host(_bf16_round((rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)))
+    ctx = Ctx(Config(num_layers=n, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv,
+                     head_dim=d, kv_capacity=T, kv_dtype=ffi.KV_BF16))
+    layer[0] = 0
+    dq, dq_f32 = dqb, dq
+    wall_ms, ev_ms = _timed(ctx, lib, step, steps, warmup)
+    res["attention_bf16_query_us_per_chunk"] = ev_ms * 1e3
+    dq = dq_f32
+    ctx.close()
 
     # The same chunk behind a context of 32768 cached positions (a long prompt taken in chunks):
     # the rows now share 1040 cache blocks instead of at most 16, which is the size at which the
@@ -242,24 +258,27 @@ def bench_prefill(steps, warmup, seed, T=512):
                      head_dim=d, kv_capacity=L0 + T, kv_dtype=ffi.KV_BF16))
     kv0 = rng.standard_normal((L0, Hkv * d), dtype=np.float32)
     ctx.kv_import(0, kv0, kv0)
-    ms, times = C.c_float(0), []
-    for i in range(4 + min(steps, 20)):
-        ctx.memory_seq_rm(L0)
-        lib.mfa_sync(ctx.h)
-        lib.mfa_timer_start(ctx.h)
-        if lib.mfa_prefill_attn_dev(ctx.h, 0, T, dq.ptr, dg.ptr, dk.ptr, dv.ptr, do.ptr) != 0:
-            raise RuntimeError(ffi.last_error())
-        lib.mfa_timer_stop(ctx.h, C.byref(ms))
-        if i >= 4:
-            times.append(ms.value)
-    med = sorted(times)[len(times) // 2]
     cflops = 2 * 2 * Hq * (T * L0 + T * (T + 1) // 2) * d
-    res["attention_after_32768_positions"] = {
-        "us_per_chunk": med * 1e3, "flop": cflops, "tflops": cflops / (med * 1e-3) / 1e12,
-        # q and the probabilities enter as two bf16 parts each: two matrix instructions per product
-        "matrix_tflops": 2 * cflops / (med * 1e-3) / 1e12, "pct_of_bf16_peak": 100 * 2 * cflops / (med * 1e-3) / 2.5e15}
+    # the probabilities enter as two bf16 parts, and so does a query that is not exact in bf16:
+    # matrix instructions per (score, value) product pair
+    for key, qdev, instr in (("attention_after_32768_positions", dq, 4), ("attention_after_32768_positions_bf16_query", dqb, 3)):
+        ms, times = C.c_float(0), []
+        for i in range(4 + min(steps, 20)):
+            ctx.memory_seq_rm(L0)
+            lib.mfa_sync(ctx.h)
+            lib.mfa_timer_start(ctx.h)
+            if lib.mfa_prefill_attn_dev(ctx.h, 0, T, qdev.ptr, dg.ptr, dk.ptr, dv.ptr, do.ptr) != 0:
+                raise RuntimeError(ffi.last_error())
+            lib.mfa_timer_stop(ctx.h, C.byref(ms))
+            if i >= 4:
+                times.append(ms.value)
+        med = sorted(times)[len(times) // 2]
+        res[key] = {
+            "us_per_chunk": med * 1e3, "flop": cflops, "tflops": cflops / (med * 1e-3) / 1e12,
+            "matrix_tflops": instr / 2 * cflops / (med * 1e-3) / 1e12,
+            "pct_of_bf16_peak": 100 * instr / 2 * cflops / (med * 1e-3) / 2.5e15}
     ctx.close()
-    for a in (dq, dg, dk, dv, do):
+    for a in (dq, dqb, dg, dk, dv, do):
         a.free()
 
     case = _GdnInputs(seed, 16, 32, 128, 128, T=T, zero_state=True)

@@ -101,19 +101,25 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
         fetch(std::integral_constant<int, 2>{}, 2);
         fetch(std::integral_constant<int, 3>{}, 3);
     }
+    // A bf16 cache's scores are products of the raw query, split into a bf16 high and low part, and are
+    // scaled as they leave the matrix core: a query that is exact in bf16 (what a bf16 model hands
+    // over) then has no low parts, and a wave all of whose rows are such leaves their products out.
     uint4 qr[RG][W::QREGS];
+    bool q_exact = true;
     int64_t limit[RG], limit_min[RG], limit_max[RG];
     bool full[RG];
 #pragma unroll
     for (int r = 0; r < RG; r++) {
         const RowGroup rows{kvh, hg0 + r, hpk, Hq, n_tok, kv_len0};
-        W::load_q_regs(qr[r], q, lane, rows, qscale);
+        W::load_q_regs(qr[r], q, lane, rows, W::kScaleAfter ? 1.0f : qscale);
+        q_exact = q_exact && W::q_low_parts_zero(qr[r]);
         limit[r] = rows.limit(n);
         limit_min[r] = rows.limit_min();
         // a group wholly past the chunk's rows sees nothing
         limit_max[r] = rows.valid(0) ? rows.limit_max() : 0;
         full[r] = rows.full();
     }
+    q_exact = __all(q_exact);
     int64_t wave_max = limit_max[0];
 #pragma unroll
     for (int r = 1; r < RG; r++) wave_max = limit_max[r] > wave_max ? limit_max[r] : wave_max;
@@ -136,8 +142,13 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
         uint4 kreg[NLOAD];
 #pragma unroll
         for (int i = 0; i < NLOAD; i++) kreg[i] = cur[i * 64 + lane];
+        if (q_exact) {
 #pragma unroll
-        for (int r = 0; r < RG; r++) W::scores_reg(kreg, qr[r], sc[r]);
+            for (int r = 0; r < RG; r++) W::template scores_reg<true>(kreg, qr[r], sc[r]);
+        } else {
+#pragma unroll
+            for (int r = 0; r < RG; r++) W::template scores_reg<false>(kreg, qr[r], sc[r]);
+        }
     };
     auto finish = [&](int64_t b, const uint4 *cur, const typename W::Scores (&sc)[RG]) __attribute__((always_inline)) {
         uint4 p[RG][W::P_U4];
@@ -145,6 +156,10 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
         for (int r = 0; r < RG; r++) {
             float x[NX];
             W::unpack(sc[r], x);
+            if constexpr (W::kScaleAfter) {
+#pragma unroll
+                for (int e = 0; e < NX; e++) x[e] *= qscale;
+            }
             if (!full[r] || (b + 1) * W::BLK > limit_min[r]) {  // a block some row must not see in full
 #pragma unroll
                 for (int e = 0; e < NX; e++)

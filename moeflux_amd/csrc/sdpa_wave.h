@@ -169,6 +169,9 @@ template <int D> struct Wave<uint16_t, D> {
         }
     }
 
+    // HI_ONLY: the query's low parts are all zero (a query that is exact in bf16), so their
+    // products are left out; the result is the same number.
+    template <bool HI_ONLY = false>
     __device__ static void scores_reg(const uint4 (&kreg)[NLOAD], const uint4 (&qr)[QREGS], Scores &sc) {
         sc.s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
         sc.s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -178,10 +181,19 @@ template <int D> struct Wave<uint16_t, D> {
             for (int sub = 0; sub < 2; sub++) {
                 const bf16x8 a = as_bf16x8(kreg[2 * s + sub]);
                 sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s]), sc.s[sub], 0, 0, 0);
-                sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s + 1]), sc.s[sub], 0, 0, 0);
+                if constexpr (!HI_ONLY)
+                    sc.s[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, as_bf16x8(qr[2 * s + 1]), sc.s[sub], 0, 0, 0);
             }
         }
     }
+    // whether every low part of this lane's query operands is zero
+    __device__ static bool q_low_parts_zero(const uint4 (&qr)[QREGS]) {
+        unsigned any = 0;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++) any |= (qr[2 * s + 1].x | qr[2 * s + 1].y | qr[2 * s + 1].z | qr[2 * s + 1].w) & 0x7fff7fffu;
+        return any == 0;
+    }
+    static constexpr bool kScaleAfter = true;   // scores leave the matrix core unscaled (prompt-chunk kernel)
 
     // One 1 KiB piece of K (16 positions x the 32 channels of k-step s) against the query
     // operands in registers: the piece's share of S^T[16 positions, 16 rows].
@@ -286,6 +298,7 @@ template <int D> struct Wave<float, D> {
         }
     }
 
+    template <bool HI_ONLY = false>   // an f32 query has no parts
     __device__ static void scores_reg(const uint4 (&kreg)[NLOAD], const uint4 (&qr)[QREGS], Scores &sc) {
         sc.s = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -298,6 +311,9 @@ template <int D> struct Wave<float, D> {
             sc.s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, sc.s, 0, 0, 0);
         }
     }
+
+    __device__ static bool q_low_parts_zero(const uint4 (&)[QREGS]) { return false; }
+    static constexpr bool kScaleAfter = false;   // the query carries the scale
 
     // One 1 KiB piece of K (16 positions x the 16 channels of k-step s).
     __device__ static f32x4 score_step(uint4 kpiece, const uint4 (&qr)[QREGS], int s, f32x4 acc) {

@@ -340,3 +340,34 @@ def test_error_paths_leave_the_context_usable(mfa, oracle):
         assert c.lib.mfa_sdpa_decode(c.h, 1, None, None, None) == ffi.ERR_INVALID
         # still works after all of that
         assert rel_err(c.sdpa_decode(1, q, g), oracle.sdpa(3, Hq, Hkv, d, q, g, k, v)) <= TOL_F32
+
+
+@pytest.mark.parametrize("L0", [0, 1000])
+def test_prefill_attn_query_exact_in_bf16_skips_nothing_that_counts(mfa, oracle, L0):
+    """The chunk kernel leaves out the products of the query's low bf16 parts in a wave all of whose
+    rows are exact in bf16.  One element of one row made inexact sends that row's wave down the
+    general path: every other row, those of the same wave included, must come out bit for bit as in
+    the run where the whole query is exact; both runs agree with the oracle."""
+    Hq, Hkv, d, T = 32, 4, 128, 256
+    rng = np.random.default_rng(77 + L0)
+    k = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)))
+    v = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)))
+    q = oracle.bf16_to_f32(oracle.f32_to_bf16((rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)))
+    g = rng.standard_normal((T, Hq * d)).astype(np.float32)
+    q2 = q.copy()
+    tok, head = 100, 3
+    q2[tok, head * d + 5] *= np.float32(1 + 2.0 ** -12)      # no longer a bf16 value
+    assert not np.array_equal(oracle.bf16_to_f32(oracle.f32_to_bf16(q2)), q2)
+    outs = []
+    for qq in (q, q2):
+        ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, qq, g, k, v).reshape(T, Hq * d)
+        with _full_ctx(mfa, Hq, Hkv, d, L0 + T, bf16=True) as c:
+            if L0:
+                c.kv_import(0, k[:L0], v[:L0])
+            outs.append(c.prefill_attn(0, qq, g, k[L0:], v[L0:]))
+        assert rel_err(outs[-1], ref) <= 1e-4
+    a, b = (o.reshape(T, Hq, d) for o in outs)
+    same = np.ones((T, Hq), bool)
+    same[tok, head] = False
+    assert np.array_equal(a[same], b[same])
+    assert not np.array_equal(a[tok, head], b[tok, head])
