@@ -256,7 +256,8 @@ __global__ __launch_bounds__(256) void gdn_chunk_post_kernel(
 static constexpr int kWyMinTokens = 48;
 
 static size_t chunk_common_elems(int Hk, int Hv, int dk, int dv, int T) {
-    return (size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 3 * (size_t)Hv + (size_t)Hk);
+    // (a multiple of 4 floats: the blocked form's arrays behind it are read and written 16 bytes at a time)
+    return ((size_t)T * (2 * (size_t)Hk * dk + 2 * (size_t)Hv * dv + 3 * (size_t)Hv + (size_t)Hk) + 3) / 4 * 4;
 }
 
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T) {
