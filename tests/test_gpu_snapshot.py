@@ -166,11 +166,19 @@ def test_snapshot_larger_than_the_staging_buffer(mfa, oracle):
             c.set_linear_weights(layer, case.conv_w, case.a_log, case.dt_bias, case.norm_w)
             c.linear_state_import(layer, case.conv_state * (layer + 1), case.ssm_state)
         probe = rng.standard_normal(8 * d, dtype=np.float32)
-        c.sdpa_decode(7, probe, probe)
-        free0 = mem_free()
+
+        def settled_free():
+            # the runtime returns a freed buffer some commands after the last one that used it
+            best = 0
+            for _ in range(8):
+                c.sdpa_decode(7, probe, probe)
+                c.sync()
+                best = max(best, mem_free())
+            return best
+
+        free0 = settled_free()
         blob = c.state_save()
-        c.sdpa_decode(7, probe, probe)
-        assert mem_free() >= free0 - (8 << 20)
+        assert settled_free() >= free0 - (8 << 20)
         want = bytearray(blob[:40])
         for layer in range(8):
             if layer in lens:
@@ -184,7 +192,5 @@ def test_snapshot_larger_than_the_staging_buffer(mfa, oracle):
         c.memory_clear()
         c.state_load(blob)
         assert [c.kv_len(layer) for layer in (1, 3, 5, 7)] == [21000, 42000, 84000, 10500]
-        # the runtime returns a freed buffer once another command has followed the last one that used it
-        c.sdpa_decode(7, probe, probe)
-        assert mem_free() >= free0 - (256 << 20) - (8 << 20)
+        assert settled_free() >= free0 - (256 << 20) - (8 << 20)
         assert c.state_save() == blob
