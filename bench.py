@@ -491,10 +491,10 @@ def bench_matvec(steps, warmup, seed):
             for i, od in enumerate(shapes):
                 tw = DeviceArray((int(lib.mfa_matvec_tiled_words(od, idim)),), np.uint32)
                 keep.append(tw)
-                if lib.mfa_matvec_tile_weights_dev(ctx.h, od, idim, specs[i].w_packed, tw.ptr) != 0:
+                if lib.mfa_matvec_tile_weights_dev(ctx.h, od, idim, specs[i].w_packed, specs[i].scales, specs[i].biases, tw.ptr) != 0:
                     raise RuntimeError(ffi.last_error())
                 sp = specs[i]
-                tspecs[i] = ffi.mfa_matvec_spec(tw.ptr, sp.scales, sp.biases, sp.x, sp.out, od, idim)
+                tspecs[i] = ffi.mfa_matvec_spec(tw.ptr, None, None, sp.x, sp.out, od, idim)
             tsets.append(tspecs)
 
         def tstep(i, tsets=tsets, n=len(shapes)):

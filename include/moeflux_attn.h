@@ -162,17 +162,19 @@ typedef struct mfa_matvec_spec {
  * 16-byte aligned (MFA_ERR_INVALID otherwise); scales and biases may start anywhere,
  * rows of them on 16-byte boundaries are read faster. */
 int mfa_dequant_matvec_4bit_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs);
-/* The same products over weights re-ordered once at load time (the reference uploads its weight
+/* The same products over a matrix re-ordered once at load time (the reference uploads its weight
  * file once, weights.rs / WeightFile; on a discrete GPU that upload is the place to re-order):
- * for every 16 rows and every 1024 inputs the bytes a wave requests, in request order, so that
- * every request is one contiguous KiB.  mfa_matvec_tiled_words gives the size of the re-ordered
- * copy in 32-bit words (rows padded to 16, inputs to 1024; negative on a bad shape),
- * mfa_matvec_tile_weights_dev writes it (device to device, on the context's stream), and
- * mfa_dequant_matvec_4bit_tiled_dev takes specs whose w_packed point at such copies; scales,
- * biases, x, out and the results are those of mfa_dequant_matvec_4bit_dev. */
+ * for every 16 rows and every 1024 inputs the bytes a wave requests, in request order - the
+ * scales and biases it multiplies with, then its weights - so that a wave's requests are nine
+ * contiguous KiB.  mfa_matvec_tiled_words gives the size of the re-ordered copy in 32-bit words
+ * (rows padded to 16, inputs to 1024; negative on a bad shape), mfa_matvec_tile_weights_dev
+ * writes it from the file's three arrays (device to device, on the context's stream), and
+ * mfa_dequant_matvec_4bit_tiled_dev takes specs whose w_packed point at such copies and whose
+ * scales and biases are not read (they may be NULL); x, out and the results, bit for bit, are
+ * those of mfa_dequant_matvec_4bit_dev. */
 int64_t mfa_matvec_tiled_words(int32_t out_dim, int32_t in_dim);
 int mfa_matvec_tile_weights_dev(mfa_ctx *ctx, int32_t out_dim, int32_t in_dim, const uint32_t *w_packed,
-                                uint32_t *w_tiled);
+                                const uint16_t *scales, const uint16_t *biases, uint32_t *w_tiled);
 int mfa_dequant_matvec_4bit_tiled_dev(mfa_ctx *ctx, int32_t n, const mfa_matvec_spec *specs);
 /* Stateless host-pointer twin of dequant_matvec_4bit_cpu (cpu_matvec.rs:83-160;
  * cpu_dequant_matvec, infer.m:671).  group_size must be 64. */

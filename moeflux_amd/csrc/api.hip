@@ -1005,10 +1005,11 @@ int64_t mfa_matvec_tiled_words(int32_t out_dim, int32_t in_dim) {
     return (int64_t)matvec_tiled_words(out_dim, in_dim);
 }
 
-int mfa_matvec_tile_weights_dev(mfa_ctx *ctx, int32_t out_dim, int32_t in_dim, const uint32_t *w_packed, uint32_t *w_tiled) {
+int mfa_matvec_tile_weights_dev(mfa_ctx *ctx, int32_t out_dim, int32_t in_dim, const uint32_t *w_packed,
+                                const uint16_t *scales, const uint16_t *biases, uint32_t *w_tiled) {
     Ctx *c = as_ctx(ctx);
     if (!c) return fail(MFA_ERR_INVALID, "NULL context");
-    return launch_matvec_tile_weights(c->stream, out_dim, in_dim, w_packed, w_tiled);
+    return launch_matvec_tile_weights(c->stream, out_dim, in_dim, w_packed, scales, biases, w_tiled);
 }
 
 int mfa_dequant_matvec_4bit(int32_t out_dim, int32_t in_dim, int32_t group_size, const uint32_t *w_packed,

@@ -120,7 +120,10 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
     const Product q = mv_product_of(sp, tl, t);
 
     mv_u32x4 w[TILES][STEPS];   // row n of tile T, 32-input chunk 4 S + g of step S
-    mv_u32x4 q0[TILES], q1[TILES];   // groups 16 wave .. + 15 of that row: scales in lanes g < 2, biases in the others
+    // The scales (lanes g < 2) or biases (the others) of row n for the wave's 16 groups.  From the file's
+    // order: q0 groups 16 wave .. + 7, q1 the next eight.  TILED: q0 alone, the eight groups of this
+    // lane's parity (2 e + g % 2, e = 0 .. 7), which are the ones it uses.
+    mv_u32x4 q0[TILES], q1[TILES];
     auto fetch = [&]() __attribute__((always_inline)) {
         const int in_dim = q.in_dim, out_dim = q.out_dim;
         const int nchunk = in_dim >> 5, groups = in_dim >> 6, words = in_dim >> 3;
@@ -128,10 +131,17 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
         // come back in the order they were asked for
 #pragma unroll
         for (int T = 0; T < TILES; T++) {
-            const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
-            const uint16_t *sb = (g < 2 ? q.scales : q.biases) + (size_t)row * groups;
-            q0[T] = load_sb8<SB16>(sb, 16 * wave, groups);
-            q1[T] = load_sb8<SB16>(sb, 16 * wave + 8, groups);
+            if constexpr (TILED) {
+                const int nruns = (in_dim + 1023) >> 10, tile = (t - q.first) * TILES + T;
+                const size_t at = (((size_t)tile * nruns + (wave < nruns ? wave : 0)) * (STEPS + 1)) * 64 + lane;
+                q0[T] = *reinterpret_cast<const mv_u32x4 *>(q.w + at * 4);
+                q1[T] = q0[T];
+            } else {
+                const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
+                const uint16_t *sb = (g < 2 ? q.scales : q.biases) + (size_t)row * groups;
+                q0[T] = load_sb8<SB16>(sb, 16 * wave, groups);
+                q1[T] = load_sb8<SB16>(sb, 16 * wave + 8, groups);
+            }
         }
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
@@ -139,9 +149,10 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
 #pragma unroll
             for (int T = 0; T < TILES; T++) {
                 if constexpr (TILED) {
-                    // [tile][run of 1024 inputs][step][lane]: a wave's request is 1 KiB in one piece
+                    // [tile][run of 1024 inputs][scales and biases, then the steps][lane]: a wave's
+                    // requests are 9 KiB in one piece, each of them 1 KiB
                     const int nruns = (in_dim + 1023) >> 10, tile = (t - q.first) * TILES + T;
-                    const size_t at = (((size_t)tile * nruns + (wave < nruns ? wave : 0)) * STEPS + st) * 64 + lane;
+                    const size_t at = (((size_t)tile * nruns + (wave < nruns ? wave : 0)) * (STEPS + 1) + 1 + st) * 64 + lane;
                     w[T][st] = *reinterpret_cast<const mv_u32x4 *>(q.w + at * 4);
                 } else {
                     const int row = min(((t - q.first) * TILES + T) * 16 + n, out_dim - 1);
@@ -250,8 +261,9 @@ __device__ __forceinline__ void dequant_matvec_body(const MatvecSpecs &sp, const
         const float xg = xs_g[2 * st];
 #pragma unroll
         for (int T = 0; T < TILES; T++) {
-            const uint32_t word = st < 4 ? q0[T][st & 3] : q1[T][st & 3];
-            const float val = __builtin_bit_cast(float, (word << sh) & 0xffff0000u);
+            // file order: element 2 st + half of the wave's 16; TILED: element st of the lane's 8
+            const uint32_t word = TILED ? q0[T][st >> 1] : st < 4 ? q0[T][st & 3] : q1[T][st & 3];
+            const float val = __builtin_bit_cast(float, (word << (TILED ? ((st & 1) ? 0 : 16) : sh)) & 0xffff0000u);
             const float dsum = (d[T][0] + d[T][1]) + d[T][2];   // sum (1 + nibble/16) x over the group
             acc[T] = fmaf(val, g < 2 ? 16.f * (dsum - xg) : xg, acc[T]);   // 16 s (D - X_g)  |  b X_g
         }
@@ -277,34 +289,52 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(5, 8
     dequant_matvec_body<WAVES, SB16, 1, TILED>(sp, tl);
 }
 
-// Weights re-ordered for the kernel above, once, when a model is loaded: for every 16-row tile
-// and every run of 1024 inputs the 8 x 64 x 16 bytes its wave requests, in request order
-// (step, then lane: row lane % 16, 32-input chunk 4 (8 run + step) + lane / 16).  Rows past
-// out_dim repeat the last row, chunks past in_dim are zero.  grid (runs, tiles), 512 threads.
-__global__ __launch_bounds__(512) void matvec_tile_weights_kernel(const uint32_t *__restrict__ w, uint32_t *__restrict__ tiled,
+// Weights, scales and biases re-ordered for the kernel above, once, when a model is loaded: for every
+// 16-row tile and every run of 1024 inputs the 9 x 64 x 16 bytes its wave requests, in request order.
+// First the scales and biases: lane (n, g) gets the eight bf16 values of row n for groups
+// 16 run + 2 e + g % 2, e = 0 .. 7 (scales for g < 2, biases for the others), the ones it multiplies
+// with.  Then the weights by step, then lane: row lane % 16, 32-input chunk 4 (8 run + step) +
+// lane / 16.  Rows past out_dim repeat the last row, chunks and groups past in_dim are zero.
+// grid (runs, tiles), 576 threads.
+__global__ __launch_bounds__(576) void matvec_tile_weights_kernel(const uint32_t *__restrict__ w, const uint16_t *__restrict__ scales,
+                                                                  const uint16_t *__restrict__ biases, uint32_t *__restrict__ tiled,
                                                                   int out_dim, int in_dim) {
     const int run = blockIdx.x, tile = blockIdx.y, nruns = gridDim.x;
-    const int st = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = threadIdx.x >> 6, lane = threadIdx.x & 63;   // request 0: scales and biases; 1 .. 8: steps
     const int row = min(16 * tile + (lane & 15), out_dim - 1);
-    const int c = 4 * (8 * run + st) + (lane >> 4);
+    const int g = lane >> 4;
     mv_u32x4 v = {0u, 0u, 0u, 0u};
-    if (c < (in_dim >> 5)) v = *reinterpret_cast<const mv_u32x4 *>(w + (size_t)row * (in_dim >> 3) + 4 * c);
-    *reinterpret_cast<mv_u32x4 *>(tiled + ((((size_t)tile * nruns + run) * 8 + st) * 64 + lane) * 4) = v;
+    if (i == 0) {
+        const int groups = in_dim >> 6;
+        const uint16_t *sb = (g < 2 ? scales : biases) + (size_t)row * groups;
+        uint32_t e[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int grp = 16 * run + 2 * k + (g & 1);
+            e[k] = grp < groups ? sb[grp] : 0u;
+        }
+        v = mv_u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+    } else {
+        const int c = 4 * (8 * run + (i - 1)) + g;
+        if (c < (in_dim >> 5)) v = *reinterpret_cast<const mv_u32x4 *>(w + (size_t)row * (in_dim >> 3) + 4 * c);
+    }
+    *reinterpret_cast<mv_u32x4 *>(tiled + ((((size_t)tile * nruns + run) * 9 + i) * 64 + lane) * 4) = v;
 }
 
 size_t matvec_tiled_words(int out_dim, int in_dim) {
-    return (size_t)((out_dim + 15) / 16) * ((in_dim + 1023) / 1024) * 8 * 64 * 4;
+    return (size_t)((out_dim + 15) / 16) * ((in_dim + 1023) / 1024) * 9 * 64 * 4;
 }
 
-int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, uint32_t *tiled) {
-    if (!w || !tiled) return fail(MFA_ERR_INVALID, "matvec tiling: NULL argument");
+int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, const uint16_t *scales,
+                               const uint16_t *biases, uint32_t *tiled) {
+    if (!w || !scales || !biases || !tiled) return fail(MFA_ERR_INVALID, "matvec tiling: NULL argument");
     if (out_dim <= 0 || in_dim <= 0 || in_dim % 64 != 0)
         return fail(MFA_ERR_INVALID, "matvec tiling: out_dim %d, in_dim %d (a multiple of 64)", out_dim, in_dim);
     if ((uintptr_t)w % 16 != 0 || (uintptr_t)tiled % 16 != 0)
         return fail(MFA_ERR_INVALID, "matvec tiling: weights must be 16-byte aligned");
     if ((out_dim + 15) / 16 > 65535) return fail(MFA_ERR_SHAPE, "matvec tiling: out_dim %d too large", out_dim);
-    hipLaunchKernelGGL(matvec_tile_weights_kernel, dim3((in_dim + 1023) / 1024, (out_dim + 15) / 16), dim3(512), 0, stream,
-                       w, tiled, out_dim, in_dim);
+    hipLaunchKernelGGL(matvec_tile_weights_kernel, dim3((in_dim + 1023) / 1024, (out_dim + 15) / 16), dim3(576), 0, stream,
+                       w, scales, biases, tiled, out_dim, in_dim);
     MFA_HIP(hipGetLastError());
     return MFA_OK;
 }
@@ -319,7 +349,7 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
     int max_out = 0, max_in = 0;
     bool sb16 = true;   // scale and bias rows can be read 16 bytes at a time in every product
     for (int i = 0; i < n; i++) {
-        if (!w[i] || !scales[i] || !biases[i] || !x[i] || !out[i]) return fail(MFA_ERR_INVALID, "dequant matvec: NULL pointer in product %d", i);
+        if (!w[i] || !x[i] || !out[i] || (!tiled && (!scales[i] || !biases[i]))) return fail(MFA_ERR_INVALID, "dequant matvec: NULL pointer in product %d", i);
         if (out_dim[i] <= 0 || in_dim[i] <= 0) return fail(MFA_ERR_INVALID, "dequant matvec: non-positive shape in product %d", i);
         if (in_dim[i] % 64 != 0) return fail(MFA_ERR_INVALID, "dequant matvec: in_dim %d is not a multiple of the group size 64", in_dim[i]);
         if (in_dim[i] > 16384) return fail(MFA_ERR_SHAPE, "dequant matvec: in_dim %d > 16384 not supported", in_dim[i]);
@@ -327,7 +357,7 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
         sp.out_dim[i] = out_dim[i]; sp.in_dim[i] = in_dim[i];
         if ((uintptr_t)w[i] % 16 != 0 || (uintptr_t)x[i] % 16 != 0)
             return fail(MFA_ERR_INVALID, "dequant matvec: weights and x of product %d must be 16-byte aligned", i);
-        if ((in_dim[i] / 64) % 8 != 0 || (uintptr_t)scales[i] % 16 != 0 || (uintptr_t)biases[i] % 16 != 0) sb16 = false;
+        if (!tiled && ((in_dim[i] / 64) % 8 != 0 || (uintptr_t)scales[i] % 16 != 0 || (uintptr_t)biases[i] % 16 != 0)) sb16 = false;
         max_out = out_dim[i] > max_out ? out_dim[i] : max_out;
         max_in = in_dim[i] > max_in ? in_dim[i] : max_in;
     }

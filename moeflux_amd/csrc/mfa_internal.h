@@ -257,7 +257,8 @@ int launch_dequant_matvec_4bit(hipStream_t stream, int n, const uint32_t *const 
                                const int *out_dim, const int *in_dim, int num_cus = 256, bool tiled = false);
 // The weight order the tiled form of the kernel reads (words of the re-ordered copy, and the copy itself).
 size_t matvec_tiled_words(int out_dim, int in_dim);
-int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, uint32_t *tiled);
+int launch_matvec_tile_weights(hipStream_t stream, int out_dim, int in_dim, const uint32_t *w, const uint16_t *scales,
+                               const uint16_t *biases, uint32_t *tiled);
 // attn_prologue.hip: q/gate split, per-head norms, rotation, cache append of one token.
 int launch_attn_prologue(hipStream_t s, int kv_dtype, int Hq, int Hkv, int D, int rotary_dim, float eps, int n_tok,
                          int32_t pos, int64_t cache_pos, size_t plane_elems, const uint16_t *q_norm,

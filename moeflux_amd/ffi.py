@@ -68,7 +68,7 @@ SIGNATURES = {
     "mfa_dequant_matvec_4bit_dev": (C.c_int, [vp, C.c_int32, vp]),
     "mfa_dequant_matvec_4bit_tiled_dev": (C.c_int, [vp, C.c_int32, vp]),
     "mfa_matvec_tiled_words": (C.c_int64, [C.c_int32, C.c_int32]),
-    "mfa_matvec_tile_weights_dev": (C.c_int, [vp, C.c_int32, C.c_int32, vp, vp]),
+    "mfa_matvec_tile_weights_dev": (C.c_int, [vp, C.c_int32, C.c_int32, vp, vp, vp, vp]),
     "mfa_dequant_matvec_4bit": (C.c_int, [C.c_int32, C.c_int32, C.c_int32, vp, u16p, u16p, f32p, f32p]),
     "mfa_mla_sdpa_folded_dev": (C.c_int, [vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_float,
                                           f32p, f32p, f32p, f32p, f32p]),

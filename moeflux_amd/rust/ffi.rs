@@ -79,7 +79,7 @@ extern "C" {
     pub fn mfa_dequant_matvec_4bit_dev(ctx: *mut mfa_ctx, n: i32, specs: *const mfa_matvec_spec) -> c_int;
     pub fn mfa_dequant_matvec_4bit_tiled_dev(ctx: *mut mfa_ctx, n: i32, specs: *const mfa_matvec_spec) -> c_int;
     pub fn mfa_matvec_tiled_words(out_dim: i32, in_dim: i32) -> i64;
-    pub fn mfa_matvec_tile_weights_dev(ctx: *mut mfa_ctx, out_dim: i32, in_dim: i32, w_packed: *const u32, w_tiled: *mut u32) -> c_int;
+    pub fn mfa_matvec_tile_weights_dev(ctx: *mut mfa_ctx, out_dim: i32, in_dim: i32, w_packed: *const u32, scales: *const u16, biases: *const u16, w_tiled: *mut u32) -> c_int;
     // attention over a latent cache (MLA, folded form)
     pub fn mfa_mla_sdpa_folded_dev(ctx: *mut mfa_ctx, num_heads: i32, kv_lora_rank: i32,
         qk_rope_head_dim: i32, cache_len: i32, softmax_scale: f32, q_prime: *const f32,

@@ -146,10 +146,11 @@ def test_scale_rows_off_a_16_byte_boundary(mfa, oracle):
 
 
 def test_tiled_weights_give_the_same_products(mfa, oracle):
-    """Weights re-ordered on the device (mfa_matvec_tile_weights_dev) and multiplied with
-    mfa_dequant_matvec_4bit_tiled_dev: the same results, bit for bit, as the file order gives, for
-    ragged row counts, input widths that do not fill a run of 1024, and products of different
-    widths in one launch; the re-ordered copy itself is checked against the layout's definition."""
+    """Weights, scales and biases re-ordered on the device (mfa_matvec_tile_weights_dev) and multiplied
+    with mfa_dequant_matvec_4bit_tiled_dev, whose specs carry no scales or biases: the same results, bit
+    for bit, as the file order gives, for ragged row counts, input widths that do not fill a run of 1024,
+    and products of different widths in one launch; the re-ordered copy itself is checked against the
+    layout's definition."""
     from moeflux_amd import Config, ffi
     from moeflux_amd.hip import DeviceArray
     rng = np.random.default_rng(10)
@@ -167,24 +168,35 @@ def test_tiled_weights_give_the_same_products(mfa, oracle):
             dw, ds, db, dx = (DeviceArray.from_host(a) for a in (packed, sc, bi, x))
             words = int(lib.mfa_matvec_tiled_words(od, idim))
             tiles, runs = (od + 15) // 16, (idim + 1023) // 1024
-            assert words == tiles * runs * 8 * 64 * 4
+            assert words == tiles * runs * 9 * 64 * 4
             dt = DeviceArray((words,), np.uint32)
-            assert lib.mfa_matvec_tile_weights_dev(c.h, od, idim, dw.ptr, dt.ptr) == 0, ffi.last_error()
+            assert lib.mfa_matvec_tile_weights_dev(c.h, od, idim, dw.ptr, ds.ptr, db.ptr, dt.ptr) == 0, ffi.last_error()
             do, dto = DeviceArray((od,), np.float32, zero=True), DeviceArray((od,), np.float32, zero=True)
             keep += [dw, ds, db, dx, dt]
             outs.append(do)
             touts.append(dto)
             specs[i] = ffi.mfa_matvec_spec(dw.ptr, ds.ptr, db.ptr, dx.ptr, do.ptr, od, idim)
-            tspecs[i] = ffi.mfa_matvec_spec(dt.ptr, ds.ptr, db.ptr, dx.ptr, dto.ptr, od, idim)
-            if i in (0, 4):   # the layout: [tile][run][step][lane] x 4 words
+            tspecs[i] = ffi.mfa_matvec_spec(dt.ptr, None, None, dx.ptr, dto.ptr, od, idim)
+            if i in (0, 4):   # the layout: [tile][run][scales and biases, then 8 steps][lane] x 4 words
                 c.sync()
-                t = dt.to_host().reshape(tiles, runs, 8, 64, 4)
+                rec = dt.to_host().reshape(tiles, runs, 9, 64, 4)
+                t = rec[:, :, 1:]
                 shape4 = (tiles, runs, 8, 64)
                 rows = np.broadcast_to(np.minimum(16 * np.arange(tiles)[:, None, None, None] + np.arange(64)[None, None, None, :] % 16, od - 1), shape4)
                 chunk = np.broadcast_to(4 * (8 * np.arange(runs)[None, :, None, None] + np.arange(8)[None, None, :, None]) + np.arange(64)[None, None, None, :] // 16, shape4)
                 src = np.zeros((od, runs * 32, 4), np.uint32)
                 src[:, :idim // 32] = packed.reshape(od, idim // 32, 4)
                 assert np.array_equal(t, src[rows, chunk])
+                # lane (n, g): row n's values for groups 16 run + 2 e + g % 2, scales for g < 2, else biases
+                sb = rec[:, :, 0].copy().view(np.uint16).reshape(tiles, runs, 64, 8)
+                groups = idim // 64
+                both = np.zeros((2, od, runs * 16), np.uint16)
+                both[0, :, :groups], both[1, :, :groups] = sc.reshape(od, groups), bi.reshape(od, groups)
+                lanes = np.arange(64)
+                r3 = np.minimum(16 * np.arange(tiles)[:, None, None, None] + (lanes % 16)[None, None, :, None], od - 1)
+                g3 = 16 * np.arange(runs)[None, :, None, None] + 2 * np.arange(8)[None, None, None, :] + ((lanes // 16) % 2)[None, None, :, None]
+                k3 = (lanes // 32)[None, None, :, None]
+                assert np.array_equal(sb, both[np.broadcast_to(k3, sb.shape), np.broadcast_to(r3, sb.shape), np.broadcast_to(g3, sb.shape)])
         assert lib.mfa_dequant_matvec_4bit_dev(c.h, len(shapes), C.byref(specs)) == 0, ffi.last_error()
         assert lib.mfa_dequant_matvec_4bit_tiled_dev(c.h, len(shapes), C.byref(tspecs)) == 0, ffi.last_error()
         c.sync()
@@ -197,7 +209,7 @@ def test_tiled_weights_give_the_same_products(mfa, oracle):
         c.sync()
         assert np.array_equal(touts[7].to_host(), outs[7].to_host())
         assert lib.mfa_matvec_tiled_words(16, 32) < 0
-        assert lib.mfa_matvec_tile_weights_dev(c.h, 16, 64, None, keep[4].ptr) == ffi.ERR_INVALID
+        assert lib.mfa_matvec_tile_weights_dev(c.h, 16, 64, None, keep[1].ptr, keep[2].ptr, keep[4].ptr) == ffi.ERR_INVALID
 
 
 def test_matvec_errors(mfa):
