@@ -191,3 +191,27 @@ def test_cache_of_131072_positions_bf16(mfa, oracle):
         c.kv_import(0, k, v)
         out = c.sdpa_decode(0, q, g)
     assert rel_err(out, ref) <= 1e-4
+
+
+@pytest.mark.parametrize("Hq,Hkv,d,bf16", [(32, 2, 256, True), (32, 4, 128, True), (8, 2, 64, True), (8, 2, 64, False)])
+def test_shares_of_a_single_unit(mfa, oracle, Hq, Hkv, d, bf16):
+    """Where a ring of loads is more than one unit's K (these shapes), a share of one unit is streamed
+    as one ring holding its K and its V: forced plans that give every workgroup exactly one unit, one
+    unit or two, and a last unit that is only partly filled, against the oracle and against a single
+    split."""
+    unit = 128 if (bf16 and d == 64) else 64      # positions of a unit of the plan
+    tol = 1e-4 if bf16 else 1e-5
+    for L, splits in ((unit * 6, 6), (unit * 6 + 17, 7), (unit * 9, 6), (unit - 14, 1), (unit * 3 - 1, 64)):
+        q, g, k, v = sdpa_random_inputs(L + splits, Hq, Hkv, d, L, bf16=bf16)
+        kf = oracle.bf16_to_f32(k) if bf16 else k
+        vf = oracle.bf16_to_f32(v) if bf16 else v
+        ref = oracle.sdpa(L, Hq, Hkv, d, q, g, k, v)
+        with _ctx(mfa, num_layers=1, full_attn_interval=1, num_attn_heads=Hq, num_kv_heads=Hkv, head_dim=d,
+                  kv_capacity=L, kv_dtype=1 if bf16 else 0) as c:
+            c.kv_import(0, kf, vf)
+            c.set_num_splits(splits)
+            out = c.sdpa_decode(0, q, g)
+            c.set_num_splits(1)
+            one = c.sdpa_decode(0, q, g)
+        assert rel_err(out, ref) <= tol, (L, splits)
+        assert rel_err(out, one) <= tol, (L, splits)

@@ -91,15 +91,21 @@ def test_prefill_attn_short_chunks_random_shapes(mfa, oracle):
                                                 (32, 4, 128, 1100, 50, True), (32, 16, 64, 2100, 0, True),
                                                 (32, 16, 64, 2050, 3, False), (4, 1, 64, 4200, 100, True),
                                                 (2, 1, 128, 4100, 0, False)])
-def test_prefill_attn_shapes(mfa, oracle, Hq, Hkv, d, T, L0, bf16):
+@pytest.mark.parametrize("q_exact", [False, True])
+def test_prefill_attn_shapes(mfa, oracle, Hq, Hkv, d, T, L0, bf16, q_exact):
     """The chunk kernel (one wave per 16-row group, K/V blocks staged in LDS) over head
-    dims, group sizes, ragged row counts and one or two row groups per wave."""
+    dims, group sizes, ragged row counts and one or two row groups per wave; with a query that is
+    exact in bf16 the waves of a bf16 cache take the path without the low parts' products."""
+    if q_exact and not bf16:
+        pytest.skip("an f32 cache has one path")
     rng = np.random.default_rng(T + L0)
     k = rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)
     v = rng.standard_normal((L0 + T, Hkv * d)).astype(np.float32)
     if bf16:
         k, v = (oracle.bf16_to_f32(oracle.f32_to_bf16(a)) for a in (k, v))
     q = (rng.standard_normal((T, Hq * d)) / np.sqrt(d)).astype(np.float32)
+    if q_exact:
+        q = oracle.bf16_to_f32(oracle.f32_to_bf16(q))
     g = rng.standard_normal((T, Hq * d)).astype(np.float32)
     ref = oracle.prefill_attn(T, L0, Hq, Hkv, d, q, g, k, v).reshape(T, Hq * d)
     with _full_ctx(mfa, Hq, Hkv, d, L0 + T, bf16=bf16) as c:
