@@ -156,10 +156,9 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
         for (int r = 0; r < RG; r++) {
             float x[NX];
             W::unpack(sc[r], x);
-            if constexpr (W::kScaleAfter) {
-#pragma unroll
-                for (int e = 0; e < NX; e++) x[e] *= qscale;
-            }
+            // kScaleAfter: x is unscaled; the scale (positive) enters the row maximum once and the
+            // exponentials' arguments as a fused multiply-add
+            const float xs = W::kScaleAfter ? qscale : 1.0f;
             if (!full[r] || (b + 1) * W::BLK > limit_min[r]) {  // a block some row must not see in full
 #pragma unroll
                 for (int e = 0; e < NX; e++)
@@ -170,6 +169,7 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
             for (int e = 1; e < NX; e++) m_loc = fmaxf(m_loc, x[e]);
             m_loc = fmaxf(m_loc, lane_xor(m_loc, 16));
             m_loc = fmaxf(m_loc, lane_xor(m_loc, 32));
+            if constexpr (W::kScaleAfter) m_loc *= xs;
             // m_loc > -inf + 8 is false while the row has seen nothing, so m_ref stays
             // -inf; the exponent's reference is then 0 and every probability is 0.
             const bool move = m_loc > m_ref[r] + kLazyRescale;
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
             float e[NX], psum = 0.f;
 #pragma unroll
             for (int i = 0; i < NX; i++) {
-                e[i] = fast_exp2(x[i] - ref);  // 0 for masked positions
+                e[i] = fast_exp2(W::kScaleAfter ? fmaf(x[i], xs, -ref) : x[i] - ref);  // 0 for masked positions
                 psum += e[i];
             }
             l_run[r] = l_run[r] * alpha + psum;
