@@ -176,8 +176,7 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
                 for (int i = 0; i < 4; i++)
                     if (pos0 + i >= L) sc[i] = neg_inf();
                 float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-                mb = fmaxf(mb, lane_xor(mb, 16));
-                mb = fmaxf(mb, lane_xor(mb, 32));
+                mb = rows_max(mb);
                 // Move the reference point only when some head's maximum has moved far: weights stay
                 // below 2^kMlaLazy, and the reference point cancels in the merge.
                 float alpha = 1.f;
@@ -200,8 +199,7 @@ __global__ __launch_bounds__(kMlaHG * 128) void mla_partial_kernel(
             }
             __syncthreads();
         }
-        l_sum += lane_xor(l_sum, 16);
-        l_sum += lane_xor(l_sum, 32);
+        l_sum = rows_sum(l_sum);
         if (active && g == 0) {
             part_ml[pid * 32 + n] = m_ref;
             part_ml[pid * 32 + 16 + n] = l_sum;

@@ -408,8 +408,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
                 m_loc = fmaxf(m_loc, x[4 * c + r]);
             }
         }
-        m_loc = fmaxf(m_loc, lane_xor(m_loc, 16));
-        m_loc = fmaxf(m_loc, lane_xor(m_loc, 32));
+        m_loc = rows_max(m_loc);
         if (g == 0) sm[wave][n] = m_loc;
         lds_barrier();
         float m_new = m_run;
@@ -464,8 +463,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_partial_kernel(
     }
 
     // ---- one partial per workgroup -----------------------------------------------
-    l_run += lane_xor(l_run, 16);
-    l_run += lane_xor(l_run, 32);
+    l_run = rows_sum(l_run);
     if (g == 0) sl[wave][n] = l_run;
     const __amdgpu_buffer_rsrc_t ob = buffer_of(part_o + pid * 16 * D);
 #pragma unroll

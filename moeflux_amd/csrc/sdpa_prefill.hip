@@ -167,8 +167,7 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
             float m_loc = x[0];
 #pragma unroll
             for (int e = 1; e < NX; e++) m_loc = fmaxf(m_loc, x[e]);
-            m_loc = fmaxf(m_loc, lane_xor(m_loc, 16));
-            m_loc = fmaxf(m_loc, lane_xor(m_loc, 32));
+            m_loc = rows_max(m_loc);
             if constexpr (W::kScaleAfter) m_loc *= xs;
             // m_loc > -inf + 8 is false while the row has seen nothing, so m_ref stays
             // -inf; the exponent's reference is then 0 and every probability is 0.
@@ -265,8 +264,7 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
 #pragma unroll
         for (int r = 0; r < RG; r++) {
             float l = l_run[r];
-            l += lane_xor(l, 16);
-            l += lane_xor(l, 32);
+            l = rows_sum(l);
             l_run[r] = l;
             if (ks > 0) {
                 if (g == 0) {
@@ -309,8 +307,7 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
 #pragma unroll
         for (int r = 0; r < RG; r++) {
             float l = l_run[r];
-            l += lane_xor(l, 16);
-            l += lane_xor(l, 32);
+            l = rows_sum(l);
             l_run[r] = l;
         }
     }

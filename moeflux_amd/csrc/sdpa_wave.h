@@ -17,6 +17,30 @@ static constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ inline float neg_inf() { return -__builtin_huge_valf(); }
 __device__ inline float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
+// Maximum / sum of a value over the four lanes l % 16 + 16 g, g = 0 .. 3, in every one of them.
+// v_permlane16_swap / v_permlane32_swap (vector ALU, no trip through the LDS crossbar) exchange the odd
+// rows of 16 lanes (the upper 32 lanes) of their first register with the even rows (the lower 32) of
+// the second: given the same value in both, a lane then holds its own value in one register and that
+// of lane l ^ 16 (l ^ 32) in the other, and the sum adds the two numbers a lane exchange would.
+// As inline assembly with two registers of their own: given one value for both operands, the
+// builtin's two results come out as one register.  (The instruction reads its operands two wait
+// states after a vector ALU write at the earliest.)
+__device__ inline void rows_swap16(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ inline void rows_swap32(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ inline float rows_max(float v) {
+    float a = v, b = v;
+    rows_swap16(a, b);
+    a = b = fmaxf(a, b);
+    rows_swap32(a, b);
+    return fmaxf(a, b);
+}
+__device__ inline float rows_sum(float v) {
+    float a = v, b = v;
+    rows_swap16(a, b);
+    a = b = a + b;
+    rows_swap32(a, b);
+    return a + b;
+}
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // (a, b) -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32)
