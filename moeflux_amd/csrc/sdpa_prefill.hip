@@ -53,6 +53,10 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
     __shared__ uint4 kv[NBUF][KS][BLK_U4];
     __shared__ float s_m[KS][RW][RG][16], s_l[KS][RW][RG][16];
 
+    // The query operands of the first wave set pass to the others (same rows; requested from memory
+    // once) through the last staging buffer, which the walk first writes in its second iteration.
+    static_assert(KS == 1 || RW * RG * W::QREGS * 64 <= KS * BLK_U4, "the query operands fit a staging buffer");
+    uint4 (*s_q)[64] = reinterpret_cast<uint4 (*)[64]>(&kv[NBUF - 1][0][0]);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rw = wave % RW, ks = wave / RW, tid = threadIdx.x % SET;
     const int n = lane & 15, g = lane >> 4;
@@ -111,14 +115,30 @@ __global__ __launch_bounds__(64 * RW * KS) void sdpa_prefill_kernel(
 #pragma unroll
     for (int r = 0; r < RG; r++) {
         const RowGroup rows{kvh, hg0 + r, hpk, Hq, n_tok, kv_len0};
-        W::load_q_regs(qr[r], q, lane, rows, W::kScaleAfter ? 1.0f : qscale);
-        q_exact = q_exact && W::q_low_parts_zero(qr[r]);
+        if (KS == 1 || ks == 0) {   // uniform over the wave
+            W::load_q_regs(qr[r], q, lane, rows, W::kScaleAfter ? 1.0f : qscale);
+            if constexpr (KS > 1) {
+#pragma unroll
+                for (int i = 0; i < W::QREGS; i++) s_q[(rw * RG + r) * W::QREGS + i][lane] = qr[r][i];
+            }
+        }
         limit[r] = rows.limit(n);
         limit_min[r] = rows.limit_min();
         // a group wholly past the chunk's rows sees nothing
         limit_max[r] = rows.valid(0) ? rows.limit_max() : 0;
         full[r] = rows.full();
     }
+    if constexpr (KS > 1) {
+        __syncthreads();
+        if (ks > 0) {
+#pragma unroll
+            for (int r = 0; r < RG; r++)
+#pragma unroll
+                for (int i = 0; i < W::QREGS; i++) qr[r][i] = s_q[(rw * RG + r) * W::QREGS + i][lane];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RG; r++) q_exact = q_exact && W::q_low_parts_zero(qr[r]);
     q_exact = __all(q_exact);
     int64_t wave_max = limit_max[0];
 #pragma unroll
