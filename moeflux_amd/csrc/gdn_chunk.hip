@@ -219,9 +219,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_recur_kernel(
     for (int i = 0; i < NI; i++) *(float4 *)(srow + 64 * i) = s[i];
 }
 
-// The gated norm (shaders.metal:1337-1370), one wave per (token, head) pair, four pairs per
-// workgroup, in blocks [0, npb); blocks [npb, npb + 32) advance the conv ring: input number s
-// lives in slot s % K, so the last min(T, K) inputs of the chunk overwrite their slots.
+// The gated norm (shaders.metal:1337-1370): DV / 4 lanes per (token, head) pair, four channels per
+// lane (16-byte loads and stores), 1024 / DV pairs per workgroup, in blocks [0, npb); blocks
+// [npb, npb + 32) advance the conv ring: input number s lives in slot s % K, so the last min(T, K)
+// inputs of the chunk overwrite their slots.
 __global__ __launch_bounds__(256) void gdn_chunk_post_kernel(
     int Hv, int DV, int T, int C, int K, int64_t step, float eps, int npb, const float *__restrict__ o_raw,
     const float *__restrict__ z, const uint16_t *__restrict__ norm_w, const float *__restrict__ qkv,
@@ -236,19 +237,23 @@ __global__ __launch_bounds__(256) void gdn_chunk_post_kernel(
         }
         return;
     }
-    const int64_t pair = (int64_t)blockIdx.x * 4 + (tid >> 6);
-    if (pair >= (int64_t)T * Hv) return;
-    const int lane = tid & 63;
-    const size_t base = (size_t)pair * DV;
-    // lane l holds elements l and l + 64; the two halves are summed separately and then
-    // added, the order of the single-step kernel's norm
-    const float x0 = lane < DV ? o_raw[base + lane] : 0.f;
-    const float x1 = lane + 64 < DV ? o_raw[base + lane + 64] : 0.f;
-    const float sum = group_sum<64>(x0 * x0) + group_sum<64>(x1 * x1);
+    const int lpr = DV >> 2;                       // lanes per pair: 16 or 32
+    const int64_t pair = (int64_t)blockIdx.x * (256 / lpr) + tid / lpr;
+    const bool ok = pair < (int64_t)T * Hv;
+    const int ch = (tid % lpr) * 4;
+    const size_t base = (size_t)(ok ? pair : 0) * DV + ch;
+    const float4 x = load_f4(o_raw + base), zz = load_f4(z + base);
+    const uint2 wb = *reinterpret_cast<const uint2 *>(norm_w + ch);
+    float sum = group_sum<16>((x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w));
+    if (lpr == 32) sum += __shfl_xor(sum, 16, 64);
     const float inv = 1.0f / sqrtf(sum / (float)DV + eps);
-    if (lane < DV) out[base + lane] = x0 * inv * bf16_bits_to_f32(norm_w[lane]) * silu_f(z[base + lane]);
-    if (lane + 64 < DV)
-        out[base + lane + 64] = x1 * inv * bf16_bits_to_f32(norm_w[lane + 64]) * silu_f(z[base + lane + 64]);
+    if (!ok) return;
+    float4 y;
+    y.x = x.x * inv * bf16_bits_to_f32((uint16_t)(wb.x & 0xffffu)) * silu_f(zz.x);
+    y.y = x.y * inv * bf16_bits_to_f32((uint16_t)(wb.x >> 16)) * silu_f(zz.y);
+    y.z = x.z * inv * bf16_bits_to_f32((uint16_t)(wb.y & 0xffffu)) * silu_f(zz.z);
+    y.w = x.w * inv * bf16_bits_to_f32((uint16_t)(wb.y >> 16)) * silu_f(zz.w);
+    *reinterpret_cast<float4 *>(out + base) = y;
 }
 
 // Chunks of at least this many tokens take the blocked form on the matrix cores; shorter
@@ -309,7 +314,8 @@ int launch_gdn_chunk(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float
                                vv, gd, bg, kq, ssm, o_raw);
     }
     MFA_HIP(hipGetLastError());
-    const int npb = (int)(((int64_t)T * Hv + 3) / 4);
+    const int ppb = 1024 / dv;   // pairs per workgroup of the gated norm
+    const int npb = (int)(((int64_t)T * Hv + ppb - 1) / ppb);
     hipLaunchKernelGGL(gdn_chunk_post_kernel, dim3(npb + 32), dim3(256), 0, s, Hv, dv, T, C, K, step, eps, npb,
                        o_raw, z, w.norm_w, qkv_in, conv_ring, out);
     MFA_HIP(hipGetLastError());
