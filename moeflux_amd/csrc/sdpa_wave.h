@@ -24,9 +24,10 @@ __device__ inline float lane_xor(float v, int mask) { return __shfl_xor(v, mask,
 // of lane l ^ 16 (l ^ 32) in the other, and the sum adds the two numbers a lane exchange would.
 // As inline assembly with two registers of their own: given one value for both operands, the
 // builtin's two results come out as one register.  (The instruction reads its operands two wait
-// states after a vector ALU write at the earliest.)
-__device__ inline void rows_swap16(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-__device__ inline void rows_swap32(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+// states after a vector ALU write at the earliest; the compiler does not see into the assembly, so
+// the wait states stand on both sides of it.)
+__device__ inline void rows_swap16(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b)); }
+__device__ inline void rows_swap32(float &a, float &b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b)); }
 __device__ inline float rows_max(float v) {
     float a = v, b = v;
     rows_swap16(a, b);
