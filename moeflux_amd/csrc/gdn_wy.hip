@@ -273,21 +273,36 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
         const int kind = job / 10, idx = job % 10;
         const int I = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
         const int J = idx - I * (I + 1) / 2;
-        const float(*X)[LDK] = kind ? sQ : sK;
         wy_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (kind == 0) {
 #pragma unroll
-        for (int s = 0; s < DK / 16; s++)
-            acc = mfma4(lds_f4(&X[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc);
-        // lane (n = m, g) holds rows 16I + 4g + i of column 16J + n
-        const int col = 16 * J + m;
+            for (int s = 0; s < DK / 16; s++)
+                acc = mfma4(lds_f4(&sK[16 * I + m][16 * s + 4 * g]), lds_f4(&sK[16 * J + m][16 * s + 4 * g]), acc);
+            // lane (n = m, g) holds rows 16I + 4g + i of column 16J + n
+            const int col = 16 * J + m;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = 16 * I + 4 * g + i;
-            const float dl = sL[row] - sL[col];
-            const float d = sR[row] > col ? 0.f : __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);  // v_exp_f32: 1 ulp
-            if (kind == 0) sA[row][col] = (col < row) ? sB[row] * d * acc[i] : 0.f;
-            else  // to tile (I, J) in A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
-                Mt[((slot * 4 + I) * 4 + J) * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = (col <= row) ? d * acc[i] : 0.f;
+            for (int i = 0; i < 4; i++) {
+                const int row = 16 * I + 4 * g + i;
+                const float dl = sL[row] - sL[col];
+                const float d = sR[row] > col ? 0.f : __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);  // v_exp_f32: 1 ulp
+                sA[row][col] = (col < row) ? sB[row] * d * acc[i] : 0.f;
+            }
+        } else {
+            // the tile transposed (k^ as the A side): lane (n = m, g) then holds columns 16J + 4g + i of
+            // row 16I + n, which is this lane's 16 bytes of tile (I, J) in A-operand order
+#pragma unroll
+            for (int s = 0; s < DK / 16; s++)
+                acc = mfma4(lds_f4(&sK[16 * J + m][16 * s + 4 * g]), lds_f4(&sQ[16 * I + m][16 * s + 4 * g]), acc);
+            const int row = 16 * I + m;
+            wy_f32x4 mv;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int col = 16 * J + 4 * g + i;
+                const float dl = sL[row] - sL[col];
+                const float d = sR[row] > col ? 0.f : __builtin_amdgcn_exp2f((dl < 0.f ? dl : 0.f) * 1.4426950408889634f);
+                mv[i] = (col <= row) ? d * acc[i] : 0.f;
+            }
+            *reinterpret_cast<wy_f32x4 *>(Mt + ((slot * 4 + I) * 4 + J) * 256 + lane * 4) = mv;
         }
     }
     for (int i = tid; i < 4 * NK * 64; i += NTHR) {  // q^ tiles, before v takes its place
@@ -386,7 +401,9 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
             const float4 tu = {t4.x * cb.x, t4.y * cb.y, t4.z * cb.z, t4.w * cb.w};
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) {
-                aw4[ct] = mfma4(tw, float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, aw4[ct]);
+                // W transposed (K as the A side): lane (n = m, g) then holds columns 16c + 4g + i of
+                // token 16 tau + n, its 16 bytes of the tile in A-operand order
+                aw4[ct] = mfma4(float4{bK[s][ct][0], bK[s][ct][1], bK[s][ct][2], bK[s][ct][3]}, tw, aw4[ct]);
                 au4[ct] = mfma4(tu, float4{bV[s][ct][0], bV[s][ct][1], bV[s][ct][2], bV[s][ct][3]}, au4[ct]);
             }
         }
@@ -394,10 +411,9 @@ __global__ __launch_bounds__(DK * 4) void gdn_wy_kernel(
         for (int ct = 0; ct < NCT; ct++) {
             const wy_f32x4 aw = aw4[ct], au = au4[ct];
             const size_t tile = (slot * 4 + tau) * NK + NCT * wave + ct;
-            // U as computed; W to A-operand order: lane (row % 16) + 16 (m / 4), component m % 4
+            // U as computed (a D tile), W in A-operand order
             *reinterpret_cast<wy_f32x4 *>(Ut + tile * 256 + lane * 4) = au;
-#pragma unroll
-            for (int i = 0; i < 4; i++) Wt[tile * 256 + ((4 * g + i) + 16 * (m >> 2)) * 4 + (m & 3)] = aw[i];
+            *reinterpret_cast<wy_f32x4 *>(Wt + tile * 256 + lane * 4) = aw;
         }
     }
 }
