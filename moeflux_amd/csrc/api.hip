@@ -888,20 +888,23 @@ int mfa_token_sweep_dev(mfa_ctx *ctx, const float *full_q, const float *full_gat
     const int64_t K = c->cfg.conv_kernel_size;
     for (auto &l : c->lin) lin_batch = lin_batch && l.w.set && l.step % K == c->lin[0].step % K;
     for (auto &f : c->full) full_batch = full_batch && f.len > 0 && f.len == c->full[0].len;
+    // With both kinds in one launch each, the merge of the attention launch's partials (few splits:
+    // the layers themselves fill the machine) rides in the first workgroups of the DeltaNet launch.
+    SdpaMergeTask merge;
     if (full_batch) {
         const int n = (int)c->full.size();
         MFA_TRY(ensure_workspace(c, 1, c->full[0].len, n));
         MFA_TRY(launch_sdpa(c->stream, c->cfg.kv_dtype, c->cfg.num_attn_heads * n, c->cfg.num_kv_heads * n,
                             c->cfg.head_dim, 1, c->full[0].len, c->plane_elems, c->full[0].k, c->full[0].v,
                             full_q, full_gate, full_out, workspace(c), c->num_cus, c->forced_splits,
-                            c->partial_only));
+                            c->partial_only, lin_batch ? &merge : nullptr));
     }
     if (lin_batch) {
         LinearLayer &l0 = c->lin[0];
         MFA_TRY(launch_gdn_step(c->stream, c->cfg.linear_num_k_heads, c->cfg.linear_num_v_heads,
                                 c->cfg.linear_key_dim, c->cfg.linear_value_dim, c->cfg.conv_kernel_size,
                                 c->cfg.rms_norm_eps, l0.w, l0.conv_ring, l0.step, l0.ssm, lin_qkv, lin_z,
-                                lin_alpha, lin_beta, lin_out, (int)c->lin.size()));
+                                lin_alpha, lin_beta, lin_out, (int)c->lin.size(), &merge));
         for (auto &l : c->lin) l.step++;
     }
     for (int i = 0; i < c->cfg.num_layers; i++) {

@@ -15,6 +15,7 @@
 // The remaining kernels in this file are one-launch twins of the five
 // reference kernels for per-kernel parity tests.
 #include "gdn_device.h"
+#include "sdpa_merge.h"
 
 namespace mfa {
 
@@ -23,8 +24,8 @@ namespace mfa {
 // are [layers, ...]: the kernel offsets each pointer by blockIdx.y strides.  KC is the conv width when it is the usual 4
 // (the taps are then requested up front, ahead of the state rows), 0 for any other width.
 template <int DK, int DV, int KC>
-__global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
-    int Hk, int Hv, int K, float eps, const uint16_t *__restrict__ conv_w,
+__device__ __forceinline__ void gdn_step_body(
+    const size_t ly, int Hk, int Hv, int K, float eps, const uint16_t *__restrict__ conv_w,
     const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
     const uint16_t *__restrict__ norm_w, float *__restrict__ conv_ring, int slot_new,
     float *__restrict__ ssm, const float *__restrict__ qkv_in, const float *__restrict__ z,
@@ -44,7 +45,6 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
     const int C = 2 * Hk * DK + Hv * DV;
     const int r = tid >> 3, j = tid & 7;
     {
-        const size_t ly = blockIdx.y;
         conv_w += ly * C * K;
         a_log += ly * Hv;
         dt_bias += ly * Hv;
@@ -185,6 +185,40 @@ __global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
         const float inv_rms = __builtin_amdgcn_rsqf(sum / (float)DV + eps);
         out[(size_t)vh * DV + tid] = s_o[tid] * inv_rms * og;
     }
+}
+
+// grid (Hv, layers): workgroup (vh, ly) steps value head vh of layer ly.
+template <int DK, int DV, int KC>
+__global__ __launch_bounds__(DV * 8) void gdn_step_kernel(
+    int Hk, int Hv, int K, float eps, const uint16_t *__restrict__ conv_w,
+    const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
+    const uint16_t *__restrict__ norm_w, float *__restrict__ conv_ring, int slot_new,
+    float *__restrict__ ssm, const float *__restrict__ qkv_in, const float *__restrict__ z,
+    const float *__restrict__ alpha, const float *__restrict__ beta, float *__restrict__ out) {
+    gdn_step_body<DK, DV, KC>(blockIdx.y, Hk, Hv, K, eps, conv_w, a_log, dt_bias, norm_w, conv_ring, slot_new, ssm, qkv_in,
+                              z, alpha, beta, out);
+}
+
+// The same with a merge of split-K partials in its first rows of workgroups (grid (Hv, merge_rows +
+// layers)): the attention layers' launch of a token sweep leaves its partials to this launch, which
+// follows it on the stream, so the sweep is two launches and the merge's round trip to memory
+// passes while the first DeltaNet workgroups wait for their operands.  A wave merges one 64-output
+// unit.
+template <int DK, int DV, int KC>
+__global__ __launch_bounds__(DV * 8) void gdn_step_merge_kernel(
+    int Hk, int Hv, int K, float eps, const uint16_t *__restrict__ conv_w,
+    const float *__restrict__ a_log, const uint16_t *__restrict__ dt_bias,
+    const uint16_t *__restrict__ norm_w, float *__restrict__ conv_ring, int slot_new,
+    float *__restrict__ ssm, const float *__restrict__ qkv_in, const float *__restrict__ z,
+    const float *__restrict__ alpha, const float *__restrict__ beta, float *__restrict__ out,
+    SdpaMergeTask merge, int merge_rows) {
+    if ((int)blockIdx.y < merge_rows) {
+        const int unit = ((int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x) * (DV * 8 / 64) + (int)(threadIdx.x >> 6);
+        if (unit < merge.n_units) sdpa_merge_unit(merge, unit, threadIdx.x & 63);   // whole waves, no barrier
+        return;
+    }
+    gdn_step_body<DK, DV, KC>(blockIdx.y - merge_rows, Hk, Hv, K, eps, conv_w, a_log, dt_bias, norm_w, conv_ring, slot_new,
+                              ssm, qkv_in, z, alpha, beta, out);
 }
 
 // ---- one-launch twins of the reference kernels ------------------------------
@@ -335,7 +369,7 @@ bool gdn_shape_supported(int Hk, int Hv, int dk, int dv, int K) {
 int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps,
                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
-                    float *out, int n_layers) {
+                    float *out, int n_layers, const SdpaMergeTask *merge) {
     if (n_layers < 1 || n_layers > 65535) return fail(MFA_ERR_INVALID, "gdn_step: bad layer count %d", n_layers);
     if (!gdn_shape_supported(Hk, Hv, dk, dv, K))
         return fail(MFA_ERR_SHAPE, "gdn_step: shape Hk=%d Hv=%d dk=%d dv=%d K=%d not supported", Hk,
@@ -345,6 +379,23 @@ int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float 
     hipLaunchKernelGGL((gdn_step_kernel<DKK, DKK, KCC>), dim3(Hv, n_layers), dim3(DKK * 8), 0, s, Hk, Hv, K, eps, \
                        w.conv_w, w.a_log, w.dt_bias, w.norm_w, conv_ring, slot_new, ssm, qkv_in, z,  \
                        alpha, beta, out)
+    if (merge && merge->n_units > 0) {
+        // a wave per unit, dv / 8 waves per workgroup, Hv workgroups per row
+        const int per_row = Hv * (dv / 8);
+        const int merge_rows = (merge->n_units + per_row - 1) / per_row;
+        if (n_layers + merge_rows > 65535) return fail(MFA_ERR_INVALID, "gdn_step: bad layer count %d", n_layers);
+#define MFA_GDN_M(DKK, KCC)                                                                                       \
+    hipLaunchKernelGGL((gdn_step_merge_kernel<DKK, DKK, KCC>), dim3(Hv, merge_rows + n_layers), dim3(DKK * 8), 0, s, Hk, \
+                       Hv, K, eps, w.conv_w, w.a_log, w.dt_bias, w.norm_w, conv_ring, slot_new, ssm, qkv_in, z,   \
+                       alpha, beta, out, *merge, merge_rows)
+        if (dk == 128 && K == 4) MFA_GDN_M(128, 4);
+        else if (dk == 128) MFA_GDN_M(128, 0);
+        else if (K == 4) MFA_GDN_M(64, 4);
+        else MFA_GDN_M(64, 0);
+#undef MFA_GDN_M
+        MFA_HIP(hipGetLastError());
+        return MFA_OK;
+    }
     if (dk == 128 && K == 4) MFA_GDN(128, 4);
     else if (dk == 128) MFA_GDN(128, 0);
     else if (K == 4) MFA_GDN(64, 4);

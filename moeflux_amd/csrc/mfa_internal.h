@@ -220,10 +220,17 @@ size_t sdpa_workspace_o_elems(int Hq, int Hkv, int D, int splits, int n_tok = 1)
 size_t sdpa_workspace_ml_elems(int Hq, int Hkv, int splits, int n_tok = 1);
 // n_tok query tokens (q, gate, out: [n_tok, Hq*D]) against a cache of kv_len positions that
 // already holds them; token t attends to positions [0, kv_len - n_tok + t].  n_tok = 1 is decode.
+// A merge of split-K partials that its caller will run inside a later launch on the same stream
+// (n_units == 0: nothing deferred).  Only merges of at most 16 splits are handed over.
+struct SdpaMergeTask {
+    const float *part_o = nullptr, *part_ml = nullptr, *gate = nullptr;
+    float *out = nullptr;
+    int nsplit = 0, hpk = 0, Hq = 0, nhg = 0, D = 0, n_units = 0;
+};
 int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
-                int forced_splits, int partial_only = 0);
+                int forced_splits, int partial_only = 0, SdpaMergeTask *defer_merge = nullptr);
 // One decode token of a full-attention layer from its raw projections in two launches (the
 // attention launch norms and rotates the query itself and appends the token; the merge takes
 // the token as one more split).  len0: cache length before the call.
@@ -307,7 +314,7 @@ bool gdn_shape_supported(int Hk, int Hv, int dk, int dv, int K);
 int launch_gdn_step(hipStream_t s, int Hk, int Hv, int dk, int dv, int K, float eps,
                     const LinearWeights &w, float *conv_ring, int64_t step, float *ssm,
                     const float *qkv_in, const float *z, const float *alpha, const float *beta,
-                    float *out, int n_layers = 1);
+                    float *out, int n_layers = 1, const SdpaMergeTask *merge = nullptr);
 // gdn_chunk.hip: T tokens through one layer (three launches); scratch holds
 // gdn_chunk_scratch_elems floats.
 size_t gdn_chunk_scratch_elems(int Hk, int Hv, int dk, int dv, int T);

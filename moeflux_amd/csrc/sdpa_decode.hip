@@ -732,7 +732,8 @@ int launch_sdpa_step(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, i
 int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_tok, int64_t kv_len,
                 size_t plane_elems, const void *k_tiled, const void *v_tiled, const float *q,
                 const float *gate, float *out, const SdpaWorkspace &ws, int num_cus,
-                int forced_splits, int partial_only) {
+                int forced_splits, int partial_only, SdpaMergeTask *defer_merge) {
+    if (defer_merge) defer_merge->n_units = 0;
     if (!sdpa_shape_supported(kv_dtype, D))
         return fail(MFA_ERR_SHAPE, "sdpa: head_dim %d / kv dtype %d not supported", D, kv_dtype);
     if (n_tok <= 0 || kv_len < n_tok)
@@ -746,6 +747,10 @@ int launch_sdpa(hipStream_t stream, int kv_dtype, int Hq, int Hkv, int D, int n_
                               hpk, Hq, n_tok, kv_len - n_tok, plan, qscale, ws.part_o, ws.part_ml, NoPrologue{});
     MFA_HIP(hipGetLastError());
     if (partial_only) return MFA_OK;
+    if (defer_merge && plan.splits <= 16) {
+        *defer_merge = SdpaMergeTask{ws.part_o, ws.part_ml, gate, out, plan.splits, hpk, Hq, plan.nhg, D, n_tok * Hq * (D / 64)};
+        return MFA_OK;
+    }
     launch_merge_kernels(stream, ws.part_o, ws.part_ml, plan.splits, hpk, Hq, plan.nhg, D, n_tok, gate, out);
     MFA_HIP(hipGetLastError());
     return MFA_OK;

@@ -184,4 +184,16 @@ __device__ inline void merge_few_units(const Reader &rd, int nsplit, int kvh, in
     }
 }
 
+// One 64-output unit of a deferred merge (what a wave of sdpa_merge_few_kernel<16> does), for
+// launches that carry such a merge in workgroups of their own.
+__device__ inline void sdpa_merge_unit(const SdpaMergeTask &t, int unit, int lane) {
+    const int per_row = t.D / 64, bx = unit / per_row, by = unit % per_row;
+    const int h = bx % t.Hq, tok = bx / t.Hq;
+    const int kvh = h / t.hpk, rr = tok * t.hpk + h % t.hpk, hg = rr / 16, n = rr % 16;
+    const size_t pid0 = ((size_t)kvh * t.nhg + hg) * t.nsplit;
+    const int u = n * per_row + by;
+    const MergeOut mo{t.gate, t.out, t.hpk, t.Hq, (t.n_units / per_row) / t.Hq, t.D, t.D, nullptr, nullptr, 0, t.nhg};
+    merge_few_units<16, 1, false>(PartialsPlain(t.part_o, t.part_ml, pid0, t.D), t.nsplit, kvh, hg, u, u + 1, mo, lane);
+}
+
 }  // namespace mfa
